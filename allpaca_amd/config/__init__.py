@@ -9,6 +9,7 @@ from typing import Any, Mapping
 from .engine import EngineConfig
 from .llama import ConfigError, Llama3RopeScaling, LlamaConfig
 from .gulidra import GulidraConfig
+from .lesarax import LesaraxConfig
 from .risizen import RisizenConfig
 
 
@@ -26,7 +27,7 @@ def read_config_json(model_dir: str) -> dict:
     return d
 
 
-__all__ = ["ConfigError", "EngineConfig", "GulidraConfig", "Llama3RopeScaling", "LlamaConfig", "RisizenConfig", "read_config_json"]
+__all__ = ["ConfigError", "EngineConfig", "GulidraConfig", "LesaraxConfig", "Llama3RopeScaling", "LlamaConfig", "RisizenConfig", "read_config_json"]
 
 
 def preset(name: str) -> dict:

@@ -61,8 +61,8 @@ __global__ __launch_bounds__(256) void attn_masked_prefill_kernel(
     const bf16_t* __restrict__ q, int ldq, void* __restrict__ out, int ldo, int H, int G, int dk, int dv,
     const bf16_t* __restrict__ cache, int P, const int* __restrict__ block_table, int max_blocks,
     const int* __restrict__ positions, const int* __restrict__ row_seg, const int* __restrict__ tile_row0,
-    const int* __restrict__ tile_rows, int n_tiles, int mask, int mask_size, int sink, float scale, int key_parts,
-    int out_f32) {
+    const int* __restrict__ tile_rows, int n_tiles, int mask, int mask_size, int sink, const float* __restrict__ sinks,
+    const float* __restrict__ gate, int ldg, float scale, int key_parts, int out_f32) {
   constexpr int KROW = DKP + (DKP % 128 == 0 ? 72 : DKP % 128 == 64 ? 8 : DKP % 128 == 32 ? 40 : 104);
   __shared__ __attribute__((aligned(16))) bf16_t Ks[KT * KROW];
   __shared__ __attribute__((aligned(16))) bf16_t Vs[DVP * (KT + KPAD)];
@@ -117,7 +117,8 @@ __global__ __launch_bounds__(256) void attn_masked_prefill_kernel(
   floatx4 o[DVP / 16];
 #pragma unroll
   for (int dt = 0; dt < DVP / 16; ++dt) o[dt] = floatx4{0.f, 0.f, 0.f, 0.f};
-  float m_run = sink ? 0.f : -INFINITY, l_run = sink ? 1.f : 0.f;   // the sink is the row's first "key"
+  // the sink is the row's first "key": its score (0, or the head's learned one; in the exponent's base 2)
+  float m_run = sink ? (sinks ? sinks[h] * LOG2E : 0.f) : -INFINITY, l_run = sink ? 1.f : 0.f;
   bf16_t* pw = Ps + wave * 16 * (KT + KPAD) + li * (KT + KPAD);
   const bf16_t* krd = Ks + li * KROW + lc * 8;
   const bf16_t* vrd = Vs + li * (KT + KPAD) + lc * 8;
@@ -250,7 +251,8 @@ __global__ __launch_bounds__(256) void attn_masked_prefill_kernel(
     __syncthreads();
   }
   if (my_row < nrows) {
-    const float inv = 1.0f / l_run;
+    float inv = 1.0f / l_run;
+    if (gate) inv *= 1.0f / (1.0f + __expf(-gate[(size_t)(row0 + my_row) * ldg + h]));
     const size_t at = (size_t)(row0 + my_row) * ldo + (size_t)h * dv;
     bf16_t* orow = (bf16_t*)out + at;
 #pragma unroll
@@ -438,11 +440,14 @@ __global__ __launch_bounds__(DT) void attn_masked_decode_kernel(
   }
 }
 
-// out[row][head] = sum_s e^(m_s - M) o_s / (sink e^(-M) + sum_s e^(m_s - M) l_s),  M = max(m_s, 0 with a sink);
+// out[row][head] = sum_s e^(m_s - M) o_s / (sink e^(z - M) + sum_s e^(m_s - M) l_s),  M = max(m_s, z with a sink), z the
+// sink's score (0, or sinks[head]); times sigmoid(gate[row][head]) with a gate;
 // at most 64 parts: lane s holds part s's maximum and sum.  The parts' elements are asked for 16 parts at a time, with
 // no condition on the way (a part beyond the last one is read as the last one, with weight 0).
 __global__ __launch_bounds__(64) void attn_masked_merge_kernel(const float* __restrict__ parts, int n_parts, int H,
                                                                int dv, const int* __restrict__ rows, int sink,
+                                                               const float* __restrict__ sinks,
+                                                               const float* __restrict__ gate, int ldg,
                                                                void* __restrict__ out, int ldo, int out_f32) {
   const int ri = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const int r = rows ? rows[ri] : ri;
@@ -450,10 +455,12 @@ __global__ __launch_bounds__(64) void attn_masked_merge_kernel(const float* __re
   const float m = lane < n_parts ? p[(size_t)lane * (dv + 2)] : -INFINITY;
   const float l = lane < n_parts ? p[(size_t)lane * (dv + 2) + 1] : 0.f;
   float M = wave_max(m);
-  if (sink) M = fmaxf(M, 0.f);
+  const float z = sinks ? sinks[h] : 0.f;
+  if (sink) M = fmaxf(M, z);
   const float w = m == -INFINITY ? 0.f : __expf(m - M);
-  const float L = wave_sum(w * l) + (sink ? __expf(-M) : 0.f);
-  const float inv = 1.0f / L;
+  const float L = wave_sum(w * l) + (sink ? __expf(z - M) : 0.f);
+  float inv = 1.0f / L;
+  if (gate) inv *= 1.0f / (1.0f + __expf(-gate[(size_t)r * ldg + h]));
   for (int e0 = 0; e0 < dv; e0 += WAVE) {
     const int e = min(e0 + lane, dv - 1);
     float a = 0.f;
@@ -495,9 +502,11 @@ APC_EXPORT int apc_attention_masked_prefill_bf16(const void* q, int ldq, void* o
                                                  int dv, const void* cache, int page_tokens, const int* block_table,
                                                  int max_blocks, const int* positions, const int* row_seg,
                                                  const int* tile_row0, const int* tile_rows, int n_tiles, int mask,
-                                                 int mask_size, int sink, float scale, int key_parts, int out_f32,
+                                                 int mask_size, int sink, const float* sinks, const float* gate,
+                                                 int ldg, float scale, int key_parts, int out_f32,
                                                  hipStream_t stream) {
   if (n_tiles <= 0) return 0;
+  if ((sinks && !sink) || (gate && ldg < H)) return APC_ERR_BAD_ARG;
   int e = check_sizes(q, ldq, out, ldo, cache, H, G, dk, dv, page_tokens, mask, mask_size, scale, key_parts, out_f32);
   if (e) return e;
   n_tiles *= 2;  // halves
@@ -506,8 +515,8 @@ APC_EXPORT int apc_attention_masked_prefill_bf16(const void* q, int ldq, void* o
 #define MP_LAUNCH(DK_, DV_)                                                                                         \
   hipLaunchKernelGGL((attn_masked_prefill_kernel<DK_, DV_>), grid, block, 0, stream, (const bf16_t*)q, ldq,          \
                      out, ldo, H, G, dk, dv, (const bf16_t*)cache, page_tokens, block_table, max_blocks,             \
-                     positions, row_seg, tile_row0, tile_rows, n_tiles, mask, mask_size, sink, scale, key_parts,    \
-                     out_f32)
+                     positions, row_seg, tile_row0, tile_rows, n_tiles, mask, mask_size, sink, sinks, gate, ldg,     \
+                     scale, key_parts, out_f32)
 #define MP_VALUES(DK_)                       \
   do {                                       \
     if (dv <= 64) MP_LAUNCH(DK_, 64);        \
@@ -528,9 +537,11 @@ APC_EXPORT int apc_attention_masked_decode_bf16(const void* q, int ldq, void* ou
                                                 int dk, int dv, const void* cache, int page_tokens,
                                                 const int* block_table, int max_blocks, const int* positions,
                                                 const int* row_seg, const int* rows, int mask, int mask_size, int sink,
-                                                float scale, int n_splits, float* parts, int key_parts, int out_f32,
+                                                const float* sinks, const float* gate, int ldg, float scale,
+                                                int n_splits, float* parts, int key_parts, int out_f32,
                                                 hipStream_t stream) {
   if (n_rows <= 0) return 0;
+  if ((sinks && !sink) || (gate && ldg < H)) return APC_ERR_BAD_ARG;
   int e = check_sizes(q, ldq, out, ldo, cache, H, G, dk, dv, page_tokens, mask, mask_size, scale, key_parts, out_f32);
   if (e) return e;
   if (!apc_attention_masked_takes(H, G, dk, dv, page_tokens, key_parts)) return APC_ERR_UNSUPPORTED;
@@ -555,7 +566,7 @@ APC_EXPORT int apc_attention_masked_decode_bf16(const void* q, int ldq, void* ou
 #undef MD_LAUNCH
   APC_LAUNCH_CHECK();
   hipLaunchKernelGGL(attn_masked_merge_kernel, dim3(n_rows, H), dim3(64), 0, stream, parts, n_splits, H, dv, rows, sink,
-                     out, ldo, out_f32);
+                     sinks, gate, ldg, out, ldo, out_f32);
   APC_LAUNCH_CHECK();
   return 0;
 }

@@ -194,19 +194,22 @@ APC_EXPORT int apc_conv_state(const void* proj, int in_dtype, int ld, const floa
 // 64 anchored at key 0, online softmax in float32.
 //   the row at position pos sees keys t in [first, pos]:
 //     mask 0: first = 0;  mask 1 (window of n): first = max(0, pos - n + 1);  mask 2 (chunks of n): first = pos - pos % n
-//   s_t = (q . K[t]) * scale;  p_t = exp(s_t) / (sink + sum exp(s_t)),  sink = 1 (a key of score 0 without a value) or 0
-//   out = sum p_t V[t];  query head h reads key/value head h / (H / G).
+//   s_t = (q . K[t]) * scale;  p_t = exp(s_t) / (sink + sum exp(s_t)),  sink = 0, 1 (a key of score 0 without a value)
+//   or exp(sinks[h]) (`sinks`: a learned score per query head, not scaled)
+//   out = sum p_t V[t] (times sigmoid(gate[row][h]) with `gate`: logits [rows][>= H]);  query head h reads key/value
+//   head h / (H / G).
 // With `key_parts` = M > 1 a key of dk elements is M keys of dk / M side by side, one for each of M maps over the same
 // values: q holds H heads of dk / M elements, head j computes its scores with part j % M of the keys of kv head
 // j / (H / G) (the M heads of a group of M are the maps of one head), and `out` holds H heads of dv.
-// The running maximum starts at 0 and the running sum at 1 with a sink (the sink is the first "key"), at -inf and 0
-// without.
+// The running maximum starts at the sink's score and the running sum at 1 with a sink (the sink is the first "key"),
+// at -inf and 0 without.
 // ---------------------------------------------------------------------------
 __global__ __launch_bounds__(64) void masked_attention_plain_kernel(
     const void* __restrict__ q, int q_dtype, int ldq, void* __restrict__ out, int out_dtype, int ldo, int H, int G,
     int dk, int dv, const void* __restrict__ cache, int cache_dtype, int P, const int* __restrict__ block_table,
     int max_blocks, const int* __restrict__ positions, const int* __restrict__ row_seg, int mask, int mask_size,
-    int sink, float scale, int key_parts) {
+    int sink, const float* __restrict__ sinks, const void* __restrict__ gate, int gate_dtype, int ldg, float scale,
+    int key_parts) {
   __shared__ float qs[MAX_PER_LANE * WAVE];
   __shared__ float ps[WAVE];
   const int r = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
@@ -226,7 +229,7 @@ __global__ __launch_bounds__(64) void masked_attention_plain_kernel(
   float o[MAX_PER_LANE];
 #pragma unroll
   for (int e = 0; e < MAX_PER_LANE; ++e) o[e] = 0.f;
-  float m = sink ? 0.f : -INFINITY, l = sink ? 1.f : 0.f;
+  float m = sink ? (sinks ? sinks[h] : 0.f) : -INFINITY, l = sink ? 1.f : 0.f;
 
   for (int c = first / WAVE; c <= pos / WAVE; ++c) {
     const int t = c * WAVE + lane;
@@ -261,7 +264,8 @@ __global__ __launch_bounds__(64) void masked_attention_plain_kernel(
       }
     }
   }
-  const float inv = 1.0f / l;
+  float inv = 1.0f / l;
+  if (gate) inv *= 1.0f / (1.0f + expf(-load_f(gate, gate_dtype, (size_t)r * ldg + h)));
 #pragma unroll
   for (int e = 0; e < MAX_PER_LANE; ++e) {
     const int i = lane + e * WAVE;
@@ -273,15 +277,17 @@ APC_EXPORT int apc_masked_attention_plain(const void* q, int q_dtype, int ldq, v
                                           int n_rows, int H, int G, int dk, int dv, const void* cache, int cache_dtype,
                                           int page_tokens, const int* block_table, int max_blocks,
                                           const int* positions, const int* row_seg, int mask, int mask_size, int sink,
-                                          float scale, int key_parts, hipStream_t stream) {
+                                          const float* sinks, const void* gate, int gate_dtype, int ldg, float scale,
+                                          int key_parts, hipStream_t stream) {
   if (n_rows <= 0) return 0;
   if (H <= 0 || G <= 0 || H % G || dk <= 0 || dv <= 0 || page_tokens <= 0 || max_blocks <= 0 || mask < 0 || mask > 2 ||
-      (mask != 0 && mask_size <= 0) || key_parts < 1 || dk % key_parts || (H / G) % key_parts)
+      (mask != 0 && mask_size <= 0) || key_parts < 1 || dk % key_parts || (H / G) % key_parts || (sinks && !sink) ||
+      (gate && ldg < H))
     return APC_ERR_BAD_ARG;
   if (dk > MAX_PER_LANE * WAVE || dv > MAX_PER_LANE * WAVE || H > 65535) return APC_ERR_UNSUPPORTED;
   hipLaunchKernelGGL(masked_attention_plain_kernel, dim3(n_rows, H), dim3(64), 0, stream, q, q_dtype, ldq, out,
                      out_dtype, ldo, H, G, dk, dv, cache, cache_dtype, page_tokens, block_table, max_blocks, positions,
-                     row_seg, mask, mask_size, sink, scale, key_parts);
+                     row_seg, mask, mask_size, sink, sinks, gate, gate_dtype, ldg, scale, key_parts);
   APC_LAUNCH_CHECK();
   return 0;
 }

@@ -4,7 +4,9 @@
 //
 //   z [T][N] router logits over N = experts with matrices + identity experts (the last ones)
 //   s = softmax(z);  chosen: the K largest of s + correction (the lower index wins a tie);  weights: s of the chosen
-//   y[t] = sum_k w[t][k] * (expert e = ids[t][k] has matrices ? Wd_e (silu(Wg_e h) * (Wu_e h)) : h)
+//   y[t] = sum_k w[t][k] * (expert e = ids[t][k] has matrices ? Wd_e (a(Wg_e h, Wu_e h)) : h)
+//   a(g, u) = silu(g) * u  (`act` 0), or with g' = min(g, limit), u' = clamp(u, -limit, limit):
+//   g' * sigmoid(alpha g') * (u' + 1)  (`act` 1)
 #include "common.h"
 #include <math.h>
 
@@ -79,7 +81,8 @@ __global__ __launch_bounds__(64) void route_topk_kernel(const float* __restrict_
 __global__ __launch_bounds__(256) void routed_glu_kernel(const void* __restrict__ h, int h_dtype, int ldh,
                                                          const void* __restrict__ w_gate_up, int w_dtype, int E, int F,
                                                          int D, const int* __restrict__ ids, int K,
-                                                         void* __restrict__ act, int act_dtype) {
+                                                         void* __restrict__ act, int act_dtype, int kind, float alpha,
+                                                         float limit) {
   extern __shared__ float hs[];
   const int pair = blockIdx.x, t = pair / K;
   const int e = ids[pair];
@@ -94,7 +97,15 @@ __global__ __launch_bounds__(256) void routed_glu_kernel(const void* __restrict_
     g = fmaf(hs[i], load_f(w_gate_up, w_dtype, gate_row + i), g);
     u = fmaf(hs[i], load_f(w_gate_up, w_dtype, up_row + i), u);
   }
-  store_f(act, act_dtype, (size_t)pair * F + f, (g / (1.0f + expf(-g))) * u);
+  float a;
+  if (kind == 1) {
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit);
+    a = g / (1.0f + expf(-alpha * g)) * (u + 1.0f);
+  } else {
+    a = (g / (1.0f + expf(-g))) * u;
+  }
+  store_f(act, act_dtype, (size_t)pair * F + f, a);
 }
 
 // y[t][d] = sum_k w[t][k] * (e has matrices ? Wd_e[d] . act[t * K + k] : h[t][d]), k in order; w_down [E][D][F]
@@ -150,13 +161,14 @@ APC_EXPORT int apc_route_topk(const float* z, int ldz, const float* correction, 
 }
 
 APC_EXPORT int apc_routed_glu(const void* h, int h_dtype, int ldh, const void* w_gate_up, int w_dtype, int E, int F,
-                              int D, const int* ids, int K, void* act, int act_dtype, int n_rows, hipStream_t stream) {
+                              int D, const int* ids, int K, void* act, int act_dtype, int n_rows, int kind, float alpha,
+                              float limit, hipStream_t stream) {
   if (n_rows <= 0 || E <= 0) return 0;
-  if (F <= 0 || D <= 0 || K <= 0 || ldh < D) return APC_ERR_BAD_ARG;
+  if (F <= 0 || D <= 0 || K <= 0 || ldh < D || kind < 0 || kind > 1) return APC_ERR_BAD_ARG;
   if ((size_t)D * sizeof(float) > 64 * 1024 || (long)n_rows * K > 0x7fffffffL || ceil_div(F, 256) > 65535)
     return APC_ERR_UNSUPPORTED;
   hipLaunchKernelGGL(routed_glu_kernel, dim3(n_rows * K, ceil_div(F, 256)), dim3(256), (size_t)D * sizeof(float),
-                     stream, h, h_dtype, ldh, w_gate_up, w_dtype, E, F, D, ids, K, act, act_dtype);
+                     stream, h, h_dtype, ldh, w_gate_up, w_dtype, E, F, D, ids, K, act, act_dtype, kind, alpha, limit);
   APC_LAUNCH_CHECK();
   return 0;
 }

@@ -54,6 +54,8 @@ class StepInfo:
     host_pos0: List[int] = field(default_factory=list)
     host_slots: List[int] = field(default_factory=list)
     max_context: int = 0              # largest (pos0 + rows) of the step
+    # the embedding's output [T, D] in the run's element type, kept by a model whose plan has links that read it
+    embedded: Optional[torch.Tensor] = None
     max_rows: int = 0                 # largest segment
     decode_only: bool = False         # every segment is a single row
     # how attention kernels divide the rows: single-row segments ("decode rows") and, for longer

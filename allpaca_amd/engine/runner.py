@@ -51,7 +51,8 @@ class ModelRunner:
         self.vocab_size = model.spec.vocab_size
         # decode-only steps are replayed as HIP graphs when every part of the model allows it: a single part that
         # plans on the host (a feed-forward that gathers rows per expert, say) would be replayed with a stale plan
-        parts = [model.embedding, model.final_norm, model.head] + [p for b in model.blocks for p in b.parts.values()]
+        parts = ([model.embedding, model.final_norm, model.head] + list(getattr(model, "links", []))
+                 + [p for b in model.blocks for p in b.parts.values()])
         self.use_graphs = bool(use_graphs) and all(getattr(p, "graph_safe", False) for p in parts)
         from ..kernels import ops
         if self.rt.dtype == torch.bfloat16 and not ops.FORCE_PLAIN:

@@ -454,11 +454,13 @@ def conv_heads(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, n_heads: 
 def masked_attention_plain(q: torch.Tensor, out: torch.Tensor, n_heads: int, n_kv_heads: int, key_dim: int,
                            value_dim: int, cache: torch.Tensor, page_tokens: int, block_table: torch.Tensor,
                            positions: torch.Tensor, row_seg: torch.Tensor, mask: str, mask_size: int, sink: bool,
-                           scale: float, key_parts: int = 1) -> None:
-    _gpu(q, out, cache, block_table, positions, row_seg)
+                           scale: float, key_parts: int = 1, sinks: Optional[torch.Tensor] = None,
+                           gate: Optional[torch.Tensor] = None) -> None:
+    _gpu(q, out, cache, block_table, positions, row_seg, sinks, gate)
     ldq, ldo = _rows(q, "attention q"), _rows(out, "attention out")
     T = q.shape[0]
     _check_key_parts(n_heads, n_kv_heads, key_dim, key_parts)
+    _check_sinks_gate(sink, sinks, gate, T, n_heads)
     _need(q.shape[1] == n_heads * (key_dim // key_parts), "attention: q must be [rows, heads * key_dim / key_parts]")
     _need(out.shape == (T, n_heads * value_dim), "attention out must be [rows, heads * value_dim]")
     _split_pages(cache, n_kv_heads, key_dim, value_dim, page_tokens)
@@ -469,7 +471,15 @@ def masked_attention_plain(q: torch.Tensor, out: torch.Tensor, n_heads: int, n_k
         q.data_ptr(), _code(q), ldq, out.data_ptr(), _code(out), ldo, T, n_heads, n_kv_heads, key_dim, value_dim,
         cache.data_ptr(), _code(cache), page_tokens, block_table.data_ptr(), block_table.shape[1],
         _i32(positions, T, "positions"), _i32(row_seg, T, "row_seg"), MASKS[mask], int(mask_size), 1 if sink else 0,
+        _f32(sinks, n_heads, "sinks"), gate.data_ptr() if gate is not None else 0,
+        _code(gate) if gate is not None else 0, _rows(gate, "head gate") if gate is not None else 0,
         float(scale), int(key_parts), _stream()), "masked_attention_plain")
+
+
+def _check_sinks_gate(sink: bool, sinks, gate, T: int, n_heads: int) -> None:
+    _need(sinks is None or sink, "attention: learned sink scores need the sink")
+    _need(gate is None or (gate.dim() == 2 and gate.shape[0] == T and gate.shape[1] >= n_heads),
+          "attention: the head gate's logits must be [rows, >= heads]")
 
 
 def _check_key_parts(n_heads: int, n_kv_heads: int, key_dim: int, key_parts: int) -> None:
@@ -480,17 +490,66 @@ def _check_key_parts(n_heads: int, n_kv_heads: int, key_dim: int, key_parts: int
 
 def masked_attention(q: torch.Tensor, out: torch.Tensor, n_heads: int, n_kv_heads: int, key_dim: int, value_dim: int,
                      cache: torch.Tensor, page_tokens: int, block_table: torch.Tensor, step, mask: str = "causal",
-                     mask_size: int = 0, sink: bool = False, scale: float = 1.0, key_parts: int = 1) -> None:
+                     mask_size: int = 0, sink: bool = False, scale: float = 1.0, key_parts: int = 1,
+                     sinks: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None) -> None:
     """`key_parts` = M > 1: a cached key of `key_dim` elements is M keys of key_dim / M side by side, one for each of M
     softmax maps over the same values; q holds `n_heads` heads of key_dim / M, head j uses part j % M (M consecutive
-    heads are the maps of one head), and `out` holds n_heads heads of value_dim (float32 or the run's type)."""
+    heads are the maps of one head), and `out` holds n_heads heads of value_dim (float32 or the run's type).
+    `sinks` float32 [heads]: the sink's score per head (0 without).  `gate` [rows, >= heads] logits: head h of a row
+    leaves multiplied by sigmoid(gate[row][h])."""
     if _tuned_ok(q, cache) and out.dtype in (torch.bfloat16, torch.float32):
         from . import tuned
         if tuned.masked_attention_bf16(q, out, n_heads, n_kv_heads, key_dim, value_dim, cache, page_tokens,
-                                       block_table, step, mask, mask_size, sink, scale, key_parts):
+                                       block_table, step, mask, mask_size, sink, scale, key_parts, sinks, gate):
             return
     masked_attention_plain(q, out, n_heads, n_kv_heads, key_dim, value_dim, cache, page_tokens, block_table,
-                           step.positions, step.row_seg, mask, mask_size, sink, scale, key_parts)
+                           step.positions, step.row_seg, mask, mask_size, sink, scale, key_parts, sinks, gate)
+
+
+def rotary_pages(q: torch.Tensor, q_off: int, n_heads: int, q_dim: int, q_rot0: int, q_out: torch.Tensor,
+                 ka: torch.Tensor, ka_off: int, a_dim: int, kb: Optional[torch.Tensor], kb_off: int, b_dim: int,
+                 kb_shared: bool, k_rot0: int, v: torch.Tensor, v_off: int, value_dim: int, n_kv_heads: int, rot: int,
+                 cos_sin: Optional[torch.Tensor], step, block_table: torch.Tensor, cache: torch.Tensor,
+                 page_tokens: int) -> None:
+    """Heads put together, rotated and cached.  Query head h: q[:, q_off + h * q_dim ...], its elements
+    [q_rot0, q_rot0 + rot) rotated by the row's position, to q_out [rows, heads * q_dim] (q_out may be q).  Key of kv
+    head g: a_dim elements of ka (column ka_off + g * a_dim) followed by b_dim elements of kb (column kb_off, the same
+    for every head if `kb_shared`, else + g * b_dim); elements [k_rot0, k_rot0 + rot) of the whole rotated; into the
+    pages.  Value of kv head g: v[:, v_off + g * value_dim ...] as it is (it may be the key's own columns).  Pairs are
+    (i, i + rot/2) of the rotated range; cos_sin float32 [positions, 2, rot/2]."""
+    _gpu(q, q_out, ka, kb, v, cos_sin, block_table, cache)
+    T = q.shape[0]
+    H, G, dq, da, db, dv = int(n_heads), int(n_kv_heads), int(q_dim), int(a_dim), int(b_dim), int(value_dim)
+    ldq, ldqo, ldka, ldv = _rows(q, "q"), _rows(q_out, "q out"), _rows(ka, "keys"), _rows(v, "values")
+    ldkb = _rows(kb, "shared key part") if kb is not None else 0
+    _need(q_off + H * dq <= q.shape[1] and q_out.shape == (T, H * dq), "rotary_pages: q heads exceed the row")
+    _need(ka.shape[0] == T and v.shape[0] == T and ka_off + G * da <= ka.shape[1] and v_off + G * dv <= v.shape[1],
+          "rotary_pages: key or value heads exceed the row")
+    _need(db == 0 or (kb is not None and kb.shape[0] == T and kb_off + (1 if kb_shared else G) * db <= kb.shape[1]),
+          "rotary_pages: the second key part exceeds its row")
+    _need(rot % 2 == 0 and 0 <= q_rot0 and q_rot0 + rot <= dq and 0 <= k_rot0 and k_rot0 + rot <= da + db,
+          "rotary_pages: the rotated range must lie inside a head")
+    if rot:
+        _need(cos_sin is not None and cos_sin.dtype == torch.float32 and cos_sin.is_contiguous()
+              and cos_sin.dim() == 3 and cos_sin.shape[1] == 2 and cos_sin.shape[2] == rot // 2,
+              "cos/sin table must be float32 [positions, 2, rot/2]")
+    _split_pages(cache, G, da + db, dv, page_tokens)
+    _need(block_table.dim() == 2 and block_table.dtype == torch.int32 and block_table.is_contiguous(),
+          "block table must be contiguous int32 [segments, blocks]")
+    if (_tuned_ok(q, q_out, ka, v, cache) and (kb is None or kb.dtype == torch.bfloat16)):
+        from . import tuned
+        if tuned.rotary_pages_bf16(q, ldq, q_off, H, dq, q_rot0, q_out, ldqo, ka, ldka, ka_off, da, kb, ldkb, kb_off,
+                                   db, kb_shared, k_rot0, v, ldv, v_off, dv, G, rot, cos_sin, step, block_table, cache,
+                                   page_tokens):
+            return
+    L = _lib.load("plain")
+    _lib.check(L.apc_rotary_pages(
+        q.data_ptr(), _code(q), ldq, q_off, H, dq, q_rot0, q_out.data_ptr(), _code(q_out), ldqo,
+        ka.data_ptr(), _code(ka), ldka, ka_off, da, kb.data_ptr() if kb is not None else 0,
+        _code(kb) if kb is not None else 0, ldkb, kb_off, db, 1 if kb_shared else 0, k_rot0,
+        v.data_ptr(), _code(v), ldv, v_off, dv, G, rot, cos_sin.data_ptr() if rot else 0,
+        _i32(step.positions, T, "positions"), _i32(step.row_seg, T, "row_seg"), block_table.data_ptr(),
+        block_table.shape[1], cache.data_ptr(), _code(cache), page_tokens, T, _stream()), "rotary_pages")
 
 
 def streams_step(x: torch.Tensor, n_streams: int, y: Optional[torch.Tensor] = None,
@@ -689,18 +748,26 @@ def prepare_experts(gate_up: torch.Tensor, down: torch.Tensor, run_dtype: torch.
     return gate_up.contiguous(), down.contiguous()
 
 
+EXPERT_ACTIVATIONS = {"silu": 0, "clamped": 1}
+
+
 def routed_experts(h: torch.Tensor, w_gate_up, w_down, n_experts: int, ff: int, ids: torch.Tensor,
-                   weights: torch.Tensor, top: int, y: torch.Tensor) -> None:
+                   weights: torch.Tensor, top: int, y: torch.Tensor, activation: str = "silu", alpha: float = 1.0,
+                   limit: float = 0.0) -> None:
     """y[t] = sum_k weights[t][k] * expert ids[t][k] (h[t]); experts 0 .. n_experts-1 are gated units
-    Wd (silu(Wg h) * (Wu h)) with w_gate_up [n_experts, 2 * ff, width] (gate rows, then up rows) and w_down
-    [n_experts, width, ff]; ids from n_experts on are identity experts.  y float32 [rows, width]."""
+    Wd a(Wg h, Wu h) with w_gate_up [n_experts, 2 * ff, width] (gate rows, then up rows) and w_down
+    [n_experts, width, ff]; ids from n_experts on are identity experts.  y float32 [rows, width].
+    `activation` "silu": a(g, u) = silu(g) * u; "clamped": g' * sigmoid(alpha g') * (u' + 1) with g' = min(g, limit),
+    u' = clamp(u, -limit, limit)."""
     T, D = h.shape
     E, F, K = int(n_experts), int(ff), int(top)
     _gpu(h, ids, weights, y)
     _need(y.dtype == torch.float32 and y.shape == (T, D), "routed_experts: y float32 [rows, width]")
+    _need(activation in EXPERT_ACTIVATIONS, f"routed_experts: activation {activation!r} is not one of {sorted(EXPERT_ACTIVATIONS)}")
+    kind = EXPERT_ACTIVATIONS[activation]
     if not isinstance(w_gate_up, torch.Tensor) and w_gate_up is not None:
         from . import tuned
-        tuned.routed_experts_bf16(h, w_gate_up, w_down, E, F, ids, weights, K, y)
+        tuned.routed_experts_bf16(h, w_gate_up, w_down, E, F, ids, weights, K, y, kind, alpha, limit)
         return
     act = torch.empty((T * K, F), dtype=h.dtype, device=h.device)
     L = _lib.load("plain")
@@ -709,7 +776,8 @@ def routed_experts(h: torch.Tensor, w_gate_up, w_down, n_experts: int, ff: int, 
         _need(w_gate_up.is_contiguous() and tuple(w_gate_up.shape) == (E, 2 * F, D) and w_down.is_contiguous()
               and tuple(w_down.shape) == (E, D, F), "routed_experts: matrices [experts, 2 ff, width] and [experts, width, ff]")
         _lib.check(L.apc_routed_glu(h.data_ptr(), _code(h), _rows(h, "h"), w_gate_up.data_ptr(), _code(w_gate_up), E, F,
-                                    D, _i32(ids, T * K, "ids"), K, act.data_ptr(), _code(act), T, _stream()),
+                                    D, _i32(ids, T * K, "ids"), K, act.data_ptr(), _code(act), T, kind, float(alpha),
+                                    float(limit), _stream()),
                    "routed_glu")
     _lib.check(L.apc_routed_down(act.data_ptr(), _code(act), w_down.data_ptr() if E else 0,
                                  _code(w_down) if E else 0, E, F, D, _i32(ids, T * K, "ids"),

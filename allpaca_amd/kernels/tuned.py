@@ -461,7 +461,8 @@ MASKED_DECODE_SPLITS = 64     # at most: the adding kernel takes 64 parts
 
 
 def masked_attention_bf16(q, out, n_heads, n_kv_heads, key_dim, value_dim, cache, page_tokens, block_table, step,
-                          mask: str, mask_size: int, sink: bool, scale: float, key_parts: int = 1) -> bool:
+                          mask: str, mask_size: int, sink: bool, scale: float, key_parts: int = 1, sinks=None,
+                          gate=None) -> bool:
     """Attention with a chunked or sliding mask and an optional sink on the MFMA kernels: segments of several rows on
     the tiled kernel, single rows on the kernel that cuts a row's keys into ranges.  False (nothing done) for sizes
     they do not take; the caller then runs the plain kernel."""
@@ -470,6 +471,11 @@ def masked_attention_bf16(q, out, n_heads, n_kv_heads, key_dim, value_dim, cache
     T = q.shape[0]
     L = _lib.load("tuned")
     f32 = out.dtype == torch.float32
+    if gate is not None and gate.dtype != torch.float32:
+        return False
+    _ops._check_sinks_gate(sink, sinks, gate, T, n_heads)
+    sinks_p = _ops._f32(sinks, n_heads, "sinks")
+    gate_p, ldg = (gate.data_ptr(), _ops._rows(gate, "head gate")) if gate is not None else (0, 0)
     if (not scale > 0 or ldq % 8 or ldo % 4 or not _aligned(q, cache) or out.data_ptr() % (16 if f32 else 8)
             or q.dtype != torch.bfloat16 or cache.dtype != torch.bfloat16
             or out.dtype not in (torch.bfloat16, torch.float32)
@@ -488,8 +494,8 @@ def masked_attention_bf16(q, out, n_heads, n_kv_heads, key_dim, value_dim, cache
             q.data_ptr(), ldq, out.data_ptr(), ldo, n_heads, n_kv_heads, key_dim, value_dim, cache.data_ptr(),
             page_tokens, block_table.data_ptr(), block_table.shape[1], step.positions.data_ptr(),
             step.row_seg.data_ptr(), step.tile_row0.data_ptr(), step.tile_rows.data_ptr(), step.n_tiles, code,
-            int(mask_size), 1 if sink else 0, float(scale), int(key_parts), 1 if f32 else 0, stream),
-            "attention_masked_prefill_bf16")
+            int(mask_size), 1 if sink else 0, sinks_p, gate_p, ldg, float(scale), int(key_parts), 1 if f32 else 0,
+            stream), "attention_masked_prefill_bf16")
     if step.n_decode_rows:
         n = step.n_decode_rows
         keys = min(step.max_decode_context, mask_size) if code else step.max_decode_context
@@ -500,8 +506,8 @@ def masked_attention_bf16(q, out, n_heads, n_kv_heads, key_dim, value_dim, cache
             q.data_ptr(), ldq, out.data_ptr(), ldo, n, n_heads, n_kv_heads, key_dim, value_dim, cache.data_ptr(),
             page_tokens, block_table.data_ptr(), block_table.shape[1], step.positions.data_ptr(),
             step.row_seg.data_ptr(), step.decode_rows.data_ptr() if step.decode_rows is not None else 0, code,
-            int(mask_size), 1 if sink else 0, float(scale), splits, parts.data_ptr(), int(key_parts),
-            1 if f32 else 0, stream), "attention_masked_decode_bf16")
+            int(mask_size), 1 if sink else 0, sinks_p, gate_p, ldg, float(scale), splits, parts.data_ptr(),
+            int(key_parts), 1 if f32 else 0, stream), "attention_masked_decode_bf16")
     return True
 
 
@@ -587,7 +593,7 @@ def pack_experts(gate_up: torch.Tensor, down: torch.Tensor):
 
 
 def routed_experts_bf16(h, w_gate_up: PackedExperts, w_down: PackedExperts, E: int, F: int, ids, weights, K: int,
-                        y) -> None:
+                        y, kind: int = 0, alpha: float = 1.0, limit: float = 0.0) -> None:
     """The chosen experts of every row on the MFMA kernels (pairs sorted by expert on the GPU, nothing read back)."""
     T, D = h.shape
     _ops._gpu(h, w_gate_up.data, w_down.data, ids, weights, y)
@@ -602,8 +608,17 @@ def routed_experts_bf16(h, w_gate_up: PackedExperts, w_down: PackedExperts, E: i
     act = torch.empty((n_pairs, F), dtype=torch.bfloat16, device=dev)
     ys = torch.empty((n_pairs, D), dtype=torch.float32, device=dev)
     hs = torch.empty((n_pairs, D), dtype=torch.bfloat16, device=dev) if tile_rows != 16 else None
+    gu = torch.empty((n_pairs, 2 * F), dtype=torch.float32, device=dev) if tile_rows != 16 and kind else None
     _lib.check(L.apc_routed_experts_bf16(
         h.data_ptr(), _ops._rows(h, "h"), w_gate_up.data.data_ptr(), w_down.data.data_ptr(), E, F, D,
         _ops._i32(ids, n_pairs, "ids"), _ops._f32(weights, n_pairs, "weights"), K, T, tile_rows, work.data_ptr(),
         act.data_ptr(), ys.data_ptr(), hs.data_ptr() if hs is not None else 0, y.data_ptr(), _ops._rows(y, "y"),
-        _ops._stream()), "routed_experts_bf16")
+        int(kind), float(alpha), float(limit), gu.data_ptr() if gu is not None else 0, _ops._stream()),
+        "routed_experts_bf16")
+
+
+def rotary_pages_bf16(q, ldq, q_off, H, dq, q_rot0, q_out, ldqo, ka, ldka, ka_off, da, kb, ldkb, kb_off, db, kb_shared,
+                      k_rot0, v, ldv, v_off, dv, G, rot, cos_sin, step, block_table, cache, page_tokens) -> bool:
+    """Heads put together, rotated and written into the pages on 16-byte accesses; False (nothing done) for sizes the
+    kernel does not take."""
+    return False

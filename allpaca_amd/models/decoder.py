@@ -11,7 +11,7 @@ from typing import Dict, List, Mapping, Optional
 import torch
 
 from ..config import read_config_json
-from ..parts import EMBEDDINGS, HEADS, NORMS, Block, Runtime, build_part
+from ..parts import CONNECTIONS, EMBEDDINGS, HEADS, NORMS, Block, Runtime, build_part
 from ..parts.base import CacheNeed
 from ..parts.spec import ModelSpec, ParamSpec
 from ..weights.loader import load_tensors
@@ -25,6 +25,8 @@ class DecoderModel:
         self.blocks: List[Block] = [Block(b) for b in spec.blocks]
         self.final_norm = build_part(NORMS, spec.final_norm)
         self.head = build_part(HEADS, spec.head)
+        # parts between plan entries (`PlanEntry.enter`); a model that has any keeps the embedding's output of a step
+        self.links = [build_part(CONNECTIONS, ls) for ls in spec.links]
         self.rt: Optional[Runtime] = None
         # called with (plan entry, residual) after every entry when set: a debugging aid (it is not part of a graph)
         self.layer_tap = None
@@ -36,6 +38,9 @@ class DecoderModel:
             out[self.spec.embedding.weight_prefix + name] = ps
         for b in self.blocks:
             out.update(b.param_specs())
+        for ls, link in zip(self.spec.links, self.links):
+            for name, ps in link.param_specs().items():
+                out[ls.weight_prefix + name] = ps
         for name, ps in self.final_norm.param_specs().items():
             out[self.spec.final_norm.weight_prefix + name] = ps
         for name, ps in self.head.param_specs().items():
@@ -51,6 +56,8 @@ class DecoderModel:
         self.embedding.bind(local(self.spec.embedding.weight_prefix, self.embedding), rt)
         for b in self.blocks:
             b.bind(tensors, rt)
+        for ls, link in zip(self.spec.links, self.links):
+            link.bind(local(ls.weight_prefix, link), rt)
         self.final_norm.bind(local(self.spec.final_norm.weight_prefix, self.final_norm), rt)
         if getattr(self.head, "tied", False):
             self.head.bind({}, rt, shared=self.embedding.weight)
@@ -91,6 +98,11 @@ class DecoderModel:
             self.embedding.forward_step(step, x)
         else:
             self.embedding.forward(step.tokens, x)
+        if self.links:
+            # the embedding's output in the element type the links' products read, kept with the step for all of them
+            from ..kernels import ops
+            step.embedded = torch.empty(x.shape, dtype=self.rt.dtype, device=self.rt.device)
+            ops.cast(x, step.embedded)
         return x
 
     def run_plan(self, x: torch.Tensor, step, caches, lo: int, hi: int, left):
@@ -98,7 +110,12 @@ class DecoderModel:
         None); returns what entry hi-1 left for entry hi's."""
         plan = self.spec.plan
         for i in range(lo, hi):
-            nxt = self.blocks[plan[i + 1].block].first_norm() if i + 1 < len(plan) else None
+            if plan[i].enter is not None:
+                self.links[plan[i].enter].apply(x, step.embedded)
+                left = None
+            nxt = None           # (a link ahead of the next entry changes the stream: nothing is left across it)
+            if i + 1 < len(plan) and plan[i + 1].enter is None:
+                nxt = self.blocks[plan[i + 1].block].first_norm()
             left = self.blocks[plan[i].block].run(x, step, caches[i], pre=left, next_norm=nxt)
             if self.layer_tap is not None:
                 self.layer_tap(i, x)

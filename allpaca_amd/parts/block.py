@@ -74,19 +74,78 @@ class Block:
             part.bind(local, rt)
 
 
+class NormedLeft:
+    """What a pre-norm layer with a scaled sum leaves for the next one: the next layer's first input, already
+    normalised (the sum of this layer's last output and that norm are one pass over the row)."""
+
+    def __init__(self, norm, h: torch.Tensor):
+        self.norm, self.h = norm, h
+
+
+class ScaledFirst:
+    """What such a layer shows the layer before it: the norm of its first read."""
+
+    def __init__(self, norm):
+        self.norm = norm
+
+    def rms_params(self):       # to an arrangement that folds norms into products this is no norm it can fold
+        return None
+
+
 @ARRANGEMENTS.register("pre_norm")
 class PreNorm:
-    """x += mixer(norm(x)); x += ffn(norm(x))  (crates/allpaca-core/src/model.rs:8447-8455, 8667-8696)."""
-    registries = {"mixer_norm": NORMS, "mixer": MIXERS, "ffn_norm": NORMS, "ffn": FEED_FORWARDS}
+    """x += mixer(norm(x)); x += ffn(norm(x))  (crates/allpaca-core/src/model.rs:8447-8455, 8667-8696).
+    With the role "scale" (a `scaled` connection) the sums are x += mult * mixer(norm(x)) and x += mult * ffn(norm(x)),
+    made in 32-bit by a kernel that also normalises the new x for whoever reads it next; such a layer may have no
+    feed-forward."""
+    registries = {"mixer_norm": NORMS, "mixer": MIXERS, "ffn_norm": NORMS, "ffn": FEED_FORWARDS, "scale": CONNECTIONS}
     chains_norms = True
 
     @staticmethod
     def first_norm(parts):
+        if "scale" in parts:
+            return ScaledFirst(parts["mixer_norm"]) if parts["mixer_norm"].rms_params() is not None else None
         return parts["mixer_norm"] if parts["mixer"].takes_normed_input else None
+
+    @staticmethod
+    def run_scaled(parts, x: torch.Tensor, step, cache, pre, next_norm):
+        mixer, ffn, link = parts["mixer"], parts.get("ffn"), parts["scale"]
+        rt = mixer.rt
+
+        def buffer():
+            return torch.empty(x.shape, dtype=rt.dtype, device=x.device)
+
+        def fusable(norm):
+            return norm is not None and norm.rms_params() is not None
+
+        if isinstance(pre, NormedLeft) and pre.norm is parts["mixer_norm"]:
+            h = pre.h
+        else:
+            h = buffer()
+            parts["mixer_norm"].forward(x, h)
+        y = mixer.forward(h, step, cache)
+        wanted = next_norm.norm if isinstance(next_norm, ScaledFirst) else None
+        if ffn is not None:
+            norm2 = parts["ffn_norm"]
+            h = buffer()
+            if fusable(norm2):
+                link.add(x, y, norm2, h)
+            else:
+                link.add(x, y)
+                norm2.forward(x, h)
+            y = ffn.forward(h, step)
+        if fusable(wanted):
+            h = buffer()
+            link.add(x, y, wanted, h)
+            return NormedLeft(wanted, h)
+        link.add(x, y)
+        return None
 
     @staticmethod
     def native_desc(parts):
         """The layer for the compiled executor, if it knows all four parts: a dict role -> the part's own description."""
+        if "scale" in parts or "ffn" not in parts:
+            return None
         out = {role: parts[role].native_desc() for role in ("mixer_norm", "mixer", "ffn_norm", "ffn")}
         kinds = {"mixer_norm": "rmsnorm", "mixer": "attention", "ffn_norm": "rmsnorm", "ffn": "swiglu"}
         if any(d is None or d.get("kind") != kinds[role] for role, d in out.items()):
@@ -95,6 +154,8 @@ class PreNorm:
 
     @staticmethod
     def run(parts, x: torch.Tensor, step, cache, pre=None, next_norm=None):
+        if "scale" in parts:
+            return PreNorm.run_scaled(parts, x, step, cache, pre, next_norm)
         mixer, ffn = parts["mixer"], parts["ffn"]
         if isinstance(cache, dict):      # a layer with several parts that keep a cache: each gets its own
             cache = cache.get("mixer")

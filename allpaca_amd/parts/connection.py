@@ -59,8 +59,47 @@ class HyperConnection(Part):
 
 @CONNECTIONS.register("scaled")
 class ScaledSum(Part):
-    """x <- x + mult * y: a constant of the layer, no tensors."""
+    """x <- x + mult * y: a constant of the layer, no tensors.  `add` does it in 32-bit; with a norm it also leaves
+    h = norm(new x) for the sublayer that reads x next (one pass over the row)."""
     graph_safe = True
 
     def __init__(self, mult: float = 1.0):
         self.mult = float(mult)
+
+    def bind(self, tensors: Mapping[str, torch.Tensor], rt: Runtime) -> None:
+        self.rt = rt
+        self._one = torch.ones(1, dtype=torch.float32, device=rt.device)
+        self._mult = torch.full((1,), self.mult, dtype=torch.float32, device=rt.device)
+
+    def add(self, x: torch.Tensor, y: torch.Tensor, norm: Optional[Norm] = None, h: Optional[torch.Tensor] = None) -> None:
+        if norm is None:
+            ops.streams_step(x, 1, y=y, mix=self._one, out_w=self._mult)
+            return
+        w, eps = norm.rms_params()
+        ops.streams_step(x, 1, y=y, mix=self._one, out_w=self._mult, in_w=self._one, norm_w=w, eps=eps, h=h)
+
+
+@CONNECTIONS.register("reinject")
+class InputInjection(Part):
+    """A link between plan entries: x <- W [x; x0], x0 the embedding's output of the row and W [width, 2 width] (x's
+    columns first).  The two halves of W are two products into the same float32 rows."""
+    graph_safe = True
+
+    def __init__(self, hidden_size: int, name: str = "weight"):
+        self.D, self.name = int(hidden_size), name
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        return {self.name: ParamSpec((self.D, 2 * self.D))}
+
+    def bind(self, tensors: Mapping[str, torch.Tensor], rt: Runtime) -> None:
+        self.rt = rt
+        w = to_device(tensors[self.name], rt)
+        self.w_x = ops.prepare_matrix(w[:, :self.D].contiguous(), rt.dtype)
+        self.w_x0 = ops.prepare_matrix(w[:, self.D:].contiguous(), rt.dtype)
+
+    def apply(self, x: torch.Tensor, x0: torch.Tensor) -> None:
+        """x float32 [rows, width] is replaced; x0 [rows, width] in the run's element type."""
+        h = torch.empty(x.shape, dtype=self.rt.dtype, device=x.device)
+        ops.cast(x, h)
+        ops.linear(h, self.w_x, x)
+        ops.linear(x0, self.w_x0, x, accumulate=True)

@@ -16,15 +16,15 @@ from .spec import ParamSpec
 class TokenEmbedding(Part):
     graph_safe = True
 
-    def __init__(self, vocab_size: int, hidden_size: int):
-        self.V, self.D = int(vocab_size), int(hidden_size)
+    def __init__(self, vocab_size: int, hidden_size: int, name: str = "weight"):
+        self.V, self.D, self.name = int(vocab_size), int(hidden_size), name      # `name`: the table's tensor name
 
     def param_specs(self) -> Dict[str, ParamSpec]:
-        return {"weight": ParamSpec((self.V, self.D))}
+        return {self.name: ParamSpec((self.V, self.D))}
 
     def bind(self, tensors: Mapping[str, torch.Tensor], rt: Runtime) -> None:
         self.rt = rt
-        self.weight = ops.prepare_matrix(to_device(tensors["weight"], rt), rt.dtype)
+        self.weight = ops.prepare_matrix(to_device(tensors[self.name], rt), rt.dtype)
 
     def forward(self, tokens: torch.Tensor, out: torch.Tensor) -> None:
         ops.embed_rows(self.weight, tokens, out)

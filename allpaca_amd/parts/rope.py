@@ -40,6 +40,25 @@ def inverse_frequencies(rot: int, theta: float, scaling: Optional[Mapping] = Non
     return np.where(wavelen < orig / hi, inv, np.where(wavelen > orig / lo, inv / factor, blended))
 
 
+_TABLES: dict = {}
+
+
+def rotary_table(rot: int, theta: float, rt: Runtime, scaling: Optional[Mapping] = None) -> torch.Tensor:
+    """float32 [positions, 2, rot/2] on the run's device: cosines and sines of position * inv_freq, the angles formed
+    in 64-bit.  Parts that ask for the same table share it."""
+    key = (int(rot), float(theta), repr(sorted(scaling.items())) if scaling else None, int(rt.max_positions),
+           str(rt.device))
+    t = _TABLES.get(key)
+    if t is None:
+        pos = np.arange(rt.max_positions, dtype=np.float64)[:, None]
+        ang = pos * inverse_frequencies(int(rot), float(theta), scaling)[None, :]
+        table = np.stack([np.cos(ang), np.sin(ang)], axis=1).astype(np.float32)
+        if len(_TABLES) >= 16:
+            _TABLES.clear()
+        t = _TABLES[key] = torch.from_numpy(table).to(rt.device).contiguous()
+    return t
+
+
 @POSITION_ENCODINGS.register("rope")
 class RotaryEncoding(PositionEncoding):
     graph_safe = True

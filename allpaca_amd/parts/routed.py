@@ -3,8 +3,10 @@
   z = Wr h (32-bit);  s = softmax(z) over all experts;  the `top` experts with the largest s + correction are chosen
   (`correction`: a tensor of one number an expert; it enters the choice only);  the weights are the chosen experts' s
   (divided by their sum with `renormalize`);  out = sum of weight * expert(h).
-An expert is a gated unit Wd (silu(Wg h) * (Wu h)) with tensors "<prefix><i>.gate|up|down"; the last `identity`
-outputs of the router stand for experts without tensors that return h itself.
+An expert is a gated unit Wd a(Wg h, Wu h) with tensors "<prefix><i>.gate|up|down"; the last `identity`
+outputs of the router stand for experts without tensors that return h itself.  `activation` "silu": a(g, u) =
+silu(g) * u; "clamped": g' * sigmoid(alpha g') * (u' + 1) with g' = min(g, limit), u' = clamp(u, -limit, limit).
+With `renormalize` and no correction the weights are the softmax over the chosen logits alone.
 The choice is made on the GPU and stays there: nothing is read back, so steps replay in graphs."""
 from __future__ import annotations
 
@@ -22,12 +24,17 @@ class RoutedExperts(FeedForward):
     graph_safe = True
 
     def __init__(self, hidden_size: int, intermediate_size: int, experts: int, top: int, identity: int = 0,
-                 correction: bool = True, renormalize: bool = False, names: Optional[Mapping[str, str]] = None):
+                 correction: bool = True, renormalize: bool = False, names: Optional[Mapping[str, str]] = None,
+                 activation: str = "silu", alpha: float = 1.0, limit: float = 0.0):
         self.D, self.F, self.E, self.K, self.I = (int(hidden_size), int(intermediate_size), int(experts), int(top),
                                                   int(identity))
         if self.E < 0 or self.I < 0 or not (1 <= self.K <= self.E + self.I):
             raise ValueError(f"routed experts: top {top} of {experts} + {identity} experts")
         self.correction, self.renormalize = bool(correction), bool(renormalize)
+        if activation not in ops.EXPERT_ACTIVATIONS or (activation == "clamped" and not float(limit) > 0):
+            raise ValueError(f"routed experts: activation {activation!r} (known: {sorted(ops.EXPERT_ACTIVATIONS)}; "
+                             f"the clamped unit needs a positive limit)")
+        self.activation, self.alpha, self.limit = activation, float(alpha), float(limit)
         self.names = {"router": "router", "correction": "correction", "expert": "e", "gate": "gate", "up": "up",
                       "down": "down", **dict(names or {})}
 
@@ -71,5 +78,6 @@ class RoutedExperts(FeedForward):
         weights = torch.empty((T, self.K), dtype=torch.float32, device=dev)
         ops.route_topk(z, self.correction_t, self.K, ids, weights, self.renormalize)
         y = torch.empty((T, self.D), dtype=torch.float32, device=dev)
-        ops.routed_experts(h, self.w_gate_up, self.w_down, self.E, self.F, ids, weights, self.K, y)
+        ops.routed_experts(h, self.w_gate_up, self.w_down, self.E, self.F, ids, weights, self.K, y,
+                           activation=self.activation, alpha=self.alpha, limit=self.limit)
         return y

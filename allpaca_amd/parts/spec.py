@@ -28,9 +28,12 @@ class BlockSpec:
 @dataclass(frozen=True)
 class PlanEntry:
     """One execution of a block.  `cache_of` names an earlier plan entry whose
-    cache this execution reads instead of writing one of its own."""
+    cache this execution reads instead of writing one of its own.  `enter` names
+    one of the model's `links` (`ModelSpec.links`): it is applied to the residual
+    stream, together with the embedding's output, right before this execution."""
     block: int
     cache_of: Optional[int] = None
+    enter: Optional[int] = None
 
 
 @dataclass(frozen=True)
@@ -76,9 +79,14 @@ class ModelSpec:
     # at the start, summed in front of the final norm); arrangements that read and write them with weights of their
     # own say how they are used
     streams: int = 1
+    # parts that stand between plan entries rather than inside a block (registry CONNECTIONS): each maps the residual
+    # stream and the embedding's output of a row to the row's new residual (`PlanEntry.enter` says where)
+    links: List[PartSpec] = field(default_factory=list)
 
     def validate(self) -> None:
         for i, e in enumerate(self.plan):
+            if e.enter is not None and not (0 <= e.enter < len(self.links)):
+                raise ValueError(f"plan[{i}].enter = {e.enter}, the model has {len(self.links)} links")
             if not (0 <= e.block < len(self.blocks)):
                 raise ValueError(f"plan[{i}] names block {e.block}, the model has {len(self.blocks)}")
             if e.cache_of is not None and not (0 <= e.cache_of < i):
