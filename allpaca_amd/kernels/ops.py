@@ -536,7 +536,7 @@ def rotary_pages(q: torch.Tensor, q_off: int, n_heads: int, q_dim: int, q_rot0: 
     _split_pages(cache, G, da + db, dv, page_tokens)
     _need(block_table.dim() == 2 and block_table.dtype == torch.int32 and block_table.is_contiguous(),
           "block table must be contiguous int32 [segments, blocks]")
-    if (_tuned_ok(q, q_out, ka, v, cache) and (kb is None or kb.dtype == torch.bfloat16)):
+    if _tuned_ok(q, q_out, ka, v, cache):
         from . import tuned
         if tuned.rotary_pages_bf16(q, ldq, q_off, H, dq, q_rot0, q_out, ldqo, ka, ldka, ka_off, da, kb, ldkb, kb_off,
                                    db, kb_shared, k_rot0, v, ldv, v_off, dv, G, rot, cos_sin, step, block_table, cache,

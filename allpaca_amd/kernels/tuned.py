@@ -619,6 +619,21 @@ def routed_experts_bf16(h, w_gate_up: PackedExperts, w_down: PackedExperts, E: i
 
 def rotary_pages_bf16(q, ldq, q_off, H, dq, q_rot0, q_out, ldqo, ka, ldka, ka_off, da, kb, ldkb, kb_off, db, kb_shared,
                       k_rot0, v, ldv, v_off, dv, G, rot, cos_sin, step, block_table, cache, page_tokens) -> bool:
-    """Heads put together, rotated and written into the pages on 16-byte accesses; False (nothing done) for sizes the
-    kernel does not take."""
-    return False
+    """Heads put together, rotated and written into the pages on 16-byte accesses (bfloat16 rows and pages; the second
+    key part may be float32 rows); False (nothing done) for sizes the kernel does not take."""
+    L = _lib.load("tuned")
+    T = q.shape[0]
+    if H <= 0 or G <= 0 or (kb is not None and kb.dtype not in (torch.bfloat16, torch.float32)):
+        return False
+    if not L.apc_rotary_pages_bf16_takes(ldq, q_off, dq, q_rot0, ldqo, ldka, ka_off, da, ldkb, kb_off, db, k_rot0, ldv,
+                                         v_off, dv, rot):
+        return False
+    if not _aligned(q, q_out, ka, v, cache) or (kb is not None and not _aligned(kb)) or (rot and not _aligned(cos_sin)):
+        return False
+    _lib.check(L.apc_rotary_pages_bf16(
+        q.data_ptr(), ldq, q_off, H, dq, q_rot0, q_out.data_ptr(), ldqo, ka.data_ptr(), ldka, ka_off, da,
+        kb.data_ptr() if kb is not None else 0, 1 if kb is not None and kb.dtype == torch.float32 else 0, ldkb, kb_off,
+        db, 1 if kb_shared else 0, k_rot0, v.data_ptr(), ldv, v_off, dv, G, rot, cos_sin.data_ptr() if rot else 0,
+        _ops._i32(step.positions, T, "positions"), _ops._i32(step.row_seg, T, "row_seg"), block_table.data_ptr(),
+        block_table.shape[1], cache.data_ptr(), page_tokens, T, _ops._stream()), "rotary_pages_bf16")
+    return True

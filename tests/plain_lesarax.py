@@ -131,7 +131,7 @@ def latent_mixer(h: np.ndarray, W: Dict[str, np.ndarray], p: str, m: dict, eps: 
     k_plain = rnd(c @ W[p + "uk"].T).reshape(T, H, dn)
     v = rnd(c @ W[p + "uv"].T).reshape(T, H, dv)
     k = np.concatenate([k_plain, np.broadcast_to(k_rot, (T, H, dr))], axis=-1)
-    o = sink_attention(q, k, v, m["scale"], W[p + "sink"], window=m["mask"]["size"])
+    o = sink_attention(q, k, v, m["scale"], W[p + "sink"], window=(m.get("mask") or {}).get("size"))
     o = o * sigmoid(h @ W[p + "g"].T)[:, :, None]
     return rnd(o.reshape(T, -1)) @ W[p + "o"].T
 
@@ -227,3 +227,37 @@ def random_weights(cfg: dict, seed: int, sharp: float = 1.0) -> Dict[str, np.nda
                 w = w * 2.0
         W[name] = to_bf16(w)
     return W
+
+
+# ---------------------------------------------------------------------------------------------- folders, generation
+def read_model_folder(path: str):
+    """(config dict, name -> float64 array) of a folder with config.json and model.safetensors: 8 bytes of length,
+    that many bytes of JSON (name -> dtype, shape, data_offsets), then the data."""
+    with open(os.path.join(path, "config.json")) as f:
+        cfg = json.load(f)
+    with open(os.path.join(path, "model.safetensors"), "rb") as f:
+        n = int.from_bytes(f.read(8), "little")
+        head = json.loads(f.read(n))
+        data = f.read()
+    W = {}
+    for name, e in head.items():
+        if name == "__metadata__":
+            continue
+        lo, hi = e["data_offsets"]
+        if e["dtype"] == "BF16":
+            a = (np.frombuffer(data[lo:hi], dtype="<u2").astype(np.uint32) << 16).view(np.float32)
+        elif e["dtype"] == "F32":
+            a = np.frombuffer(data[lo:hi], dtype="<f4")
+        else:
+            raise ValueError(f"{name}: element type {e['dtype']}")
+        W[name] = a.astype(np.float64).reshape(e["shape"])
+    return cfg, W
+
+
+def greedy(cfg: dict, W: Dict[str, np.ndarray], prompt, n: int) -> List[int]:
+    """The n tokens that follow `prompt` when the largest logit is taken every time (the lowest id wins a tie).  The
+    whole sequence is computed anew for every token: this implementation keeps nothing between calls."""
+    toks = list(prompt)
+    for _ in range(n):
+        toks.append(int(np.argmax(forward(cfg, W, toks)[-1])))
+    return toks[len(prompt):]
