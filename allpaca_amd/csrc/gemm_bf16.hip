@@ -47,11 +47,15 @@ struct TiledPre {
 // Rows in runs that each multiply with a matrix of their own (routed experts: the rows that chose an expert lie side by
 // side): `tiles` holds (matrix, first row, rows) of every row tile, `*n_tiles` of them, and matrix e starts
 // `w_stride` elements behind matrix e - 1.  The grid is (column tiles, most row tiles there can be); a block beyond
-// the tiles that exist leaves at once.  tiles == nullptr: one matrix for all rows.
+// the tiles that exist leaves at once.  tiles == nullptr: one matrix for all rows.  act, alpha, limit: the activation of
+// the gated unit in mode G_SWIGLU (see gated_unit_act; 0: silu(g) * u).
 struct GroupedRows {
   const int* tiles;
   const int* n_tiles;
   size_t w_stride;
+  int act = 0;
+  float alpha = 1.0f;
+  float limit = 0.0f;
 };
 
 // EVEN_K: K is a multiple of 64, so no load needs a bound check.  BM: rows of the block tile, 64 or 128.
@@ -299,7 +303,9 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(const bf16_t* __restrict
       }
       if (MODE == G_SWIGLU) {
         const int n = n0 + wn * 32 + li;
-        if (n < N) ((bf16_t*)C)[(size_t)m * ldc + n] = float_to_bf16(silu_f(acc[a][0][r]) * acc[a][1][r]);
+        if (n < N)
+          ((bf16_t*)C)[(size_t)m * ldc + n] =
+              float_to_bf16(gated_unit_act(acc[a][0][r], acc[a][1][r], grp.act, grp.alpha, grp.limit));
       } else {
 #pragma unroll
         for (int b = 0; b < 2; ++b) {
@@ -636,17 +642,17 @@ APC_EXPORT int apc_gemm_bf16(const void* A, int lda, const void* W, void* C, int
   }
 }
 
-// Rows in runs of one matrix each (see GroupedRows): mode G_SWIGLU (W, W2: gate and up; bfloat16 out) or G_STORE_F32.
-// tile_rows: 64 or 128, the rows `tiles` was cut for.
+// Rows in runs of one matrix each (see GroupedRows): mode G_SWIGLU (W, W2: gate and up; bfloat16 out; act, alpha, limit:
+// the gated unit's activation) or G_STORE_F32.  tile_rows: 64 or 128, the rows `tiles` was cut for.
 APC_EXPORT int apc_gemm_grouped_bf16(const void* A, int lda, const void* W, const void* W2, size_t w_stride, void* C,
                                      int ldc, const int* tiles, const int* n_tiles, int max_tiles, int tile_rows,
-                                     int N, int K, int mode, hipStream_t stream) {
+                                     int N, int K, int mode, int act, float alpha, float limit, hipStream_t stream) {
   if (max_tiles <= 0) return 0;
   if (N <= 0 || K <= 0 || K % 8 || lda % 8 || !tiles || !n_tiles || (tile_rows != 64 && tile_rows != 128) ||
-      (mode != G_SWIGLU && mode != G_STORE_F32) || (mode == G_SWIGLU && !W2) || max_tiles > 65535)
+      (mode != G_SWIGLU && mode != G_STORE_F32) || (mode == G_SWIGLU && !W2) || max_tiles > 65535 || act < 0 || act > 1)
     return APC_ERR_BAD_ARG;
   if (!aligned16(A) || !aligned16(W) || (W2 && !aligned16(W2))) return APC_ERR_UNSUPPORTED;
-  const GroupedRows grp{tiles, n_tiles, w_stride};
+  const GroupedRows grp{tiles, n_tiles, w_stride, act, alpha, limit};
   const int nb = mode == G_SWIGLU ? BN / 2 : BN;
   const dim3 grid(ceil_div(N, nb), max_tiles);
 #define GROUPED_LAUNCH(MODE_, EVEN_, BM_)                                                                          \

@@ -55,3 +55,13 @@ __device__ __forceinline__ floatx16 mfma32(const Frag& a, const Frag& b, floatx1
 }
 
 __device__ __forceinline__ float silu_f(float g) { return g / (1.0f + __expf(-g)); }
+// a gated unit's activation.  kind 0: silu(g) * u; kind 1, the clamped unit: g' * sigmoid(alpha g') * (u' + 1) with
+// g' = min(g, limit) and u' = clamp(u, -limit, limit)
+__device__ __forceinline__ float gated_unit_act(float g, float u, int kind, float alpha, float limit) {
+  if (kind == 1) {
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit);
+    return g / (1.0f + __expf(-alpha * g)) * (u + 1.0f);
+  }
+  return silu_f(g) * u;
+}

@@ -28,14 +28,8 @@ constexpr int TILE_ELEMS = 512;
 constexpr int MAX_EXPERTS = 1024;
 constexpr int STREAM_U = 4;       // chunks of 32 columns a wave asks for together
 
-// the gated unit's activation: kind 0 silu(g) * u; kind 1 the clamped unit
 __device__ __forceinline__ float unit_act(float g, float u, int kind, float alpha, float limit) {
-  if (kind == 1) {
-    g = fminf(g, limit);
-    u = fminf(fmaxf(u, -limit), limit);
-    return g / (1.0f + __expf(-alpha * g)) * (u + 1.0f);
-  }
-  return silu_f(g) * u;
+  return gated_unit_act(g, u, kind, alpha, limit);
 }
 
 __global__ __launch_bounds__(1024) void routed_sort_kernel(const int* __restrict__ ids, int n_pairs, int E,
@@ -242,20 +236,6 @@ __global__ __launch_bounds__(256) void routed_gather_kernel(const bf16_t* __rest
   }
 }
 
-// act[p][f] = a(gu[p][f], gu[p][F + f]) over the sorted places (float32 gate and up columns side by side)
-__global__ __launch_bounds__(256) void routed_act_kernel(const float* __restrict__ gu, int F, const int* __restrict__ tiles,
-                                                         const int* __restrict__ n_tiles, bf16_t* __restrict__ act,
-                                                         int kind, float alpha, float limit) {
-  const int ti = blockIdx.x;
-  if (ti >= *n_tiles) return;
-  const int p0 = tiles[3 * ti + 1], rows = tiles[3 * ti + 2];
-  for (int idx = blockIdx.y * 256 + threadIdx.x; idx < rows * F; idx += gridDim.y * 256) {
-    const int r = idx / F, f = idx % F;
-    const float* row = gu + (size_t)(p0 + r) * 2 * F;
-    act[(size_t)(p0 + r) * F + f] = float_to_bf16(unit_act(row[f], row[F + f], kind, alpha, limit));
-  }
-}
-
 __global__ __launch_bounds__(256) void routed_combine_kernel(const float* __restrict__ ys, const int* __restrict__ place,
                                                              const float* __restrict__ weights, int K,
                                                              const bf16_t* __restrict__ h, int ldh,
@@ -286,19 +266,18 @@ APC_EXPORT int apc_routed_max_tiles(int n_pairs, int E, int tile_rows) {
 
 extern "C" int apc_gemm_grouped_bf16(const void* A, int lda, const void* W, const void* W2, size_t w_stride, void* C,
                                      int ldc, const int* tiles, const int* n_tiles, int max_tiles, int tile_rows,
-                                     int N, int K, int mode, hipStream_t stream);
+                                     int N, int K, int mode, int act, float alpha, float limit, hipStream_t stream);
 
 // work: int32 [2 * n_pairs + 3 * max_tiles + 1] (order, place, tiles, the tiles' count); act: bfloat16 [n_pairs, F];
 // ys: float32 [n_pairs, D]; hs: bfloat16 [n_pairs, D] (tiles of 64 and 128 rows only).  tile_rows: 16, 64 or 128.
-// kind, alpha, limit: the activation (0: silu(g) * u; 1: the clamped unit, which on tiles of 64 and 128 rows needs
-// `gu`: float32 [n_pairs, 2 F], gate and up columns before the activation).
+// kind, alpha, limit: the activation (0: silu(g) * u; 1: the clamped unit), applied where gate and up are formed.
 APC_EXPORT int apc_routed_experts_bf16(const void* h, int ldh, const void* w_gate_up, const void* w_down, int E, int F,
                                        int D, const int* ids, const float* weights, int K, int n_rows, int tile_rows,
                                        int* work, void* act, float* ys, void* hs, float* y, int ldy, int kind,
-                                       float alpha, float limit, float* gu, hipStream_t stream) {
+                                       float alpha, float limit, hipStream_t stream) {
   if (n_rows <= 0) return 0;
   if (!apc_routed_bf16_takes(E, F, D)) return APC_ERR_UNSUPPORTED;
-  if (kind < 0 || kind > 1 || (kind == 1 && tile_rows != 16 && (!gu || ((uintptr_t)gu & 15u)))) return APC_ERR_BAD_ARG;
+  if (kind < 0 || kind > 1) return APC_ERR_BAD_ARG;
   if (K <= 0 || ldh < D || ldy < D || ldh % 8 || (tile_rows != 16 && tile_rows != 64 && tile_rows != 128) || !work ||
       !act || !ys || (tile_rows != 16 && (!hs || ((uintptr_t)hs & 15u))) ||
       ((uintptr_t)h & 15u) || ((uintptr_t)w_gate_up & 15u) || ((uintptr_t)w_down & 15u) || ((uintptr_t)act & 15u) ||
@@ -329,25 +308,12 @@ APC_EXPORT int apc_routed_experts_bf16(const void* h, int ldh, const void* w_gat
     APC_LAUNCH_CHECK();
     const size_t gate_elems = (size_t)ceil_div(F, 16) * ceil_div(D, 32) * TILE_ELEMS;
     const size_t down_elems = (size_t)ceil_div(D, 16) * ceil_div(F, 32) * TILE_ELEMS;
-    int e;
-    if (kind == 0) {
-      e = apc_gemm_grouped_bf16(hs, D, w_gate_up, (const bf16_t*)w_gate_up + gate_elems, 2 * gate_elems, act, F,
-                                tiles, n_tiles, max_tiles, tile_rows, F, D, /* SwiGLU */ 3, stream);
-      if (e) return e;
-    } else {
-      // gate and up as two products with float32 columns side by side, then the activation over the sorted places
-      for (int half = 0; half < 2; ++half) {
-        e = apc_gemm_grouped_bf16(hs, D, (const bf16_t*)w_gate_up + half * gate_elems, nullptr, 2 * gate_elems,
-                                  gu + (size_t)half * F, 2 * F, tiles, n_tiles, max_tiles, tile_rows, F, D,
-                                  /* float32 out */ 1, stream);
-        if (e) return e;
-      }
-      hipLaunchKernelGGL(routed_act_kernel, dim3(max_tiles, 8), dim3(256), 0, stream, gu, F, tiles, n_tiles,
-                         (bf16_t*)act, kind, alpha, limit);
-      APC_LAUNCH_CHECK();
-    }
+    int e = apc_gemm_grouped_bf16(hs, D, w_gate_up, (const bf16_t*)w_gate_up + gate_elems, 2 * gate_elems, act, F,
+                                  tiles, n_tiles, max_tiles, tile_rows, F, D, /* gated unit */ 3, kind, alpha, limit,
+                                  stream);
+    if (e) return e;
     e = apc_gemm_grouped_bf16(act, F, w_down, nullptr, down_elems, ys, D, tiles, n_tiles, max_tiles, tile_rows, D, F,
-                              /* float32 out */ 1, stream);
+                              /* float32 out */ 1, 0, 1.0f, 0.0f, stream);
     if (e) return e;
   }
   hipLaunchKernelGGL(routed_combine_kernel, dim3(n_rows), dim3(256), 0, stream, ys, place, weights, K,

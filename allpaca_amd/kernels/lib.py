@@ -80,7 +80,7 @@ SIGNATURES: Dict[str, Dict[str, list]] = {
         "apc_conv_heads_bf16": [P, I, I, I, I, I, I, P, P, I, P, I, I, P, P, P, P, I, F, I, P, P, P, I, P, I, P, I, P],
         "apc_routed_bf16_takes": [I, I, I],
         "apc_routed_max_tiles": [I, I, I],
-        "apc_routed_experts_bf16": [P, I, P, P, I, I, I, P, P, I, I, I, P, P, P, P, P, I, I, F, F, P, P],
+        "apc_routed_experts_bf16": [P, I, P, P, I, I, I, P, P, I, I, I, P, P, P, P, P, I, I, F, F, P],
         "apc_linear_attention_bf16_takes": [I, I, I, I, I, I, I],
         "apc_linear_attention_bf16": [P, I, I, I, I, I, I, I, I, P, P, I, P, P, P, I, P, P, P, P, I, P],
         "apc_attention_masked_takes": [I, I, I, I, I, I],

@@ -608,12 +608,11 @@ def routed_experts_bf16(h, w_gate_up: PackedExperts, w_down: PackedExperts, E: i
     act = torch.empty((n_pairs, F), dtype=torch.bfloat16, device=dev)
     ys = torch.empty((n_pairs, D), dtype=torch.float32, device=dev)
     hs = torch.empty((n_pairs, D), dtype=torch.bfloat16, device=dev) if tile_rows != 16 else None
-    gu = torch.empty((n_pairs, 2 * F), dtype=torch.float32, device=dev) if tile_rows != 16 and kind else None
     _lib.check(L.apc_routed_experts_bf16(
         h.data_ptr(), _ops._rows(h, "h"), w_gate_up.data.data_ptr(), w_down.data.data_ptr(), E, F, D,
         _ops._i32(ids, n_pairs, "ids"), _ops._f32(weights, n_pairs, "weights"), K, T, tile_rows, work.data_ptr(),
         act.data_ptr(), ys.data_ptr(), hs.data_ptr() if hs is not None else 0, y.data_ptr(), _ops._rows(y, "y"),
-        int(kind), float(alpha), float(limit), gu.data_ptr() if gu is not None else 0, _ops._stream()),
+        int(kind), float(alpha), float(limit), _ops._stream()),
         "routed_experts_bf16")
 
 

@@ -574,6 +574,113 @@ def gulidra_run(args) -> int:
     return 0
 
 
+# ---- the Lesarax design beside the llama decoder at equal sizes ---------------------------------------------------
+LESARAX_LIKE_KERNELS = {
+    "apc_rotary_pages_bf16": ["apc_rope_kv_write_bf16", "apc_rope_kv_write"],
+    "apc_attention_masked_prefill_bf16": ["apc_attention_prefill_bf16"],
+    "apc_attention_masked_decode_bf16": ["apc_attention_decode_bf16"],
+    "apc_routed_experts_bf16": ["apc_gemm_swiglu_bf16", "apc_skinny_swiglu_bf16", "apc_skinny_swiglu_pre_bf16"],
+    "apc_streams_step": ["apc_rmsnorm_rows"],
+    "apc_route_topk": [],
+}
+LESARAX_EXPERTS, LESARAX_TOP, LESARAX_WINDOW = 8, 2, 1024
+
+
+def lesarax_configs(size: str, context: int):
+    """Two layers that run twice in a row (four layer runs, each with pages of its own): a latent attention (latents of
+    3/8 and 1/8 of the width, heads of d unrotated and d/2 rotated key elements, values of d, a window of 1,024) and a
+    grouped attention whose values are its keys (heads of d, half of them rotated), each with routed experts (2 of 8,
+    each half as wide as the dense feed-forward: the same arithmetic a row); the llama decoder with four layers of the
+    same widths."""
+    D, H, G, d, F, V = DESIGN_SIZES[size]
+    latent = dict(heads=H, dim=d, rot_dim=d // 2, vdim=d, q_rank=3 * D // 8, kv_rank=D // 8, scale=(d + d // 2) ** -0.5,
+                  rot=dict(base=10000.0, dims=d // 2), mask=dict(size=LESARAX_WINDOW))
+    grouped = dict(heads=H, kv_heads=G, dim=d, vdim=d, scale=d ** -0.5, rot=dict(base=500000.0, dims=d // 2))
+    moe = dict(kind="moe", expert=dict(ff=F // LESARAX_TOP, limit=7.0),
+               router=dict(experts=LESARAX_EXPERTS, top=LESARAX_TOP))
+    lesarax = dict(architecture="Lesarax", vocab=V, width=D, residual_mult=0.5, norm=dict(eps=1e-6),
+                   max_positions=2 * context + 4096, loop=dict(start=0, stop=2, times=2),
+                   layers=[dict(type="latent_attention", mixer=latent, mlp=moe),
+                           dict(type="attention", mixer=grouped, mlp=moe)])
+    return {"lesarax": lesarax, "llama": design_configs(size, 4, 2 * context)["llama"]}
+
+
+def lesarax_rooflines(size, batch, context, T, points):
+    """For the kernels the design adds and their like kernels of the llama decoder: the bytes or the arithmetic of the
+    launches of a step over the measured time, as a share of the GPU's peak (8 TB/s, 2.5 PFLOP/s)."""
+    D, H, G, d, F, V = DESIGN_SIZES[size]
+    Fe, E, K, W = F // LESARAX_TOP, LESARAX_EXPERTS, LESARAX_TOP, LESARAX_WINDOW
+    dr = d // 2
+
+    def work(name, model, rows, keys_sum, keys_in_window):
+        """(bytes, flops) of all of a step's launches of entry point `name` in `model`."""
+        if name == "apc_rotary_pages_bf16":      # per run: the projected rows read, q and the pages' rows written
+            grouped = (H + G) * d + H * d + 2 * G * d
+            latent = H * (d + dr) + 2 * H * d + 2 * dr + H * (d + dr) + H * (2 * d + dr)
+            return 2 * rows * (grouped + latent) * 2, 0
+        if name in ("apc_rope_kv_write_bf16", "apc_rope_kv_write"):
+            return 4 * rows * ((H + 2 * G) * d + H * d + 2 * G * d) * 2, 0
+        if name == "apc_attention_masked_prefill_bf16":      # two runs over all earlier keys, two inside the window
+            return 0, 2 * keys_sum * H * 4 * d + 2 * keys_in_window * H * (2 * (d + dr) + 2 * d)
+        if name == "apc_attention_prefill_bf16":
+            return 0, 4 * 4 * keys_sum * H * d
+        if name == "apc_attention_masked_decode_bf16":       # keys and values of every kv head; every head has its own
+            return (2 * keys_sum * G * 2 * d + 2 * keys_in_window * H * (2 * d + dr)) * 2, 0      # in the latent runs
+        if name == "apc_attention_decode_bf16":
+            return 4 * keys_sum * G * 2 * d * 2, 0
+        if name == "apc_routed_experts_bf16":
+            used = min(E, rows * K)
+            return 4 * used * 3 * Fe * D * 2, 4 * rows * K * 3 * 2 * Fe * D
+        if name in ("apc_gemm_swiglu_bf16", "apc_skinny_swiglu_bf16", "apc_skinny_swiglu_pre_bf16"):
+            return 4 * 2 * F * D * 2, 4 * rows * 2 * 2 * F * D
+        if name == "apc_streams_step":               # y and x read, x and the next reader's 16-bit copy written
+            return 8 * rows * D * (4 + 4 + 4 + 2), 0
+        if name == "apc_rmsnorm_rows":
+            return 9 * rows * D * (4 + 2), 0
+        return None
+
+    table = {}
+    in_window = sum(min(p + 1, W) for p in range(T))
+    for phase, rows, keys_sum, kw in (("prefill", T, T * (T + 1) // 2, in_window),
+                                      ("decode", batch, batch * context, batch * min(context, W))):
+        for new, likes in LESARAX_LIKE_KERNELS.items():
+            row = {}
+            for model, names in (("lesarax", [new]), ("llama", likes)):
+                us = sum(points[model][phase + "_kernels_us"].get(n, 0.0) for n in names)
+                name = next((n for n in names if n in points[model][phase + "_kernels_us"]), None)
+                if not us or name is None:
+                    continue
+                w = work(name, model, rows, keys_sum, kw)
+                row[model] = {"us": round(us, 1)}
+                if w:
+                    row[model]["share_of_peak"] = round(max(w[0] / (us * 1e-6) / (HBM_PEAK_GBS * 1e9),
+                                                            w[1] / (us * 1e-6) / PEAK_FLOPS["bf16"]), 4)
+            if row:
+                table[f"{phase}: {new}"] = row
+    return table
+
+
+def lesarax_run(args) -> int:
+    T, batch, context = 2048, args.batch, args.context
+    out = {"metric": "Lesarax beside the llama decoder at equal sizes: prefill tok/s (one prompt of 2048 tokens) and "
+                     f"decode tok/s (batch {batch}, context {context})", "unit": "tok/s", "n_gpus": 1,
+           "dtype": args.dtype, "data": "synthetic: random N(0, 0.02) weights, uniform random token ids",
+           "config": {"layers": "(latent attention + experts, grouped attention + experts) twice in a row",
+                      "experts": LESARAX_EXPERTS, "top": LESARAX_TOP, "window": LESARAX_WINDOW, "page_tokens": 16},
+           "sizes": {}}
+    for size in args.design_sizes.split(","):
+        cfgs = lesarax_configs(size, context)
+        points = {m: design_point(c, args.dtype, batch, context, args.steps, args.warmup, T) for m, c in cfgs.items()}
+        out["sizes"][size] = {
+            "shape": dict(zip(("width", "heads", "kv_heads", "head_size", "ff", "vocab"), DESIGN_SIZES[size])),
+            **points,
+            "prefill_lesarax_over_llama": round(points["lesarax"]["prefill_tok_s"] / points["llama"]["prefill_tok_s"], 3),
+            "decode_lesarax_over_llama": round(points["lesarax"]["decode_tok_s"] / points["llama"]["decode_tok_s"], 3),
+            "like_kernels": lesarax_rooflines(size, batch, context, T, points)}
+    print(json.dumps(out), flush=True)
+    return 0
+
+
 def design_point(cfg_json, dtype, batch, context, steps, warmup, T):
     """Prefill tok/s (one prompt of T tokens in one step), decode tok/s (batch x context, graphs) and the time of
     every kernel in an eager prefill step and an eager decode step of one model."""
@@ -739,7 +846,7 @@ def main() -> int:
                     help="for profiling: only the decode steps at --batch (as --no-points), only the 2,048-token "
                          "prefill (prints its figures as the line's value), or only the sampler over the preset's "
                          "vocabulary (microseconds a step's rows take on the GPU and on the host)")
-    ap.add_argument("--design", choices=["risizen", "gulidra"], default=None,
+    ap.add_argument("--design", choices=["risizen", "gulidra", "lesarax"], default=None,
                     help="instead of the default workload: the named design beside the llama decoder at equal sizes "
                          "(--design-sizes), prefill and decode throughput and the times of their like kernels")
     ap.add_argument("--design-sizes", default="1b,8b", help="with --design: sizes of the comparison, of " + ",".join(DESIGN_SIZES))
@@ -760,6 +867,8 @@ def main() -> int:
 
     if args.design == "gulidra":
         return gulidra_run(args)
+    if args.design == "lesarax":
+        return lesarax_run(args)
     if args.design:
         return design_run(args)
     if args.kernel_times:
