@@ -84,6 +84,61 @@ def _rot(m: Mapping[str, Any], where: str) -> Tuple[int, float]:
     return dims, base
 
 
+def sizes_from_tensors(d: Mapping[str, Any], shapes: Mapping[str, Tuple[int, ...]]) -> Mapping[str, Any]:
+    """config.json with the sizes it leaves out filled in from the shapes of the stored tensors (`embed`,
+    `l<i>.mix.*`, `l<i>.mlp.*`).  A size the file names is left as it is: a disagreement shows when the weights load."""
+    def rows(name: str) -> Optional[int]:
+        shape = shapes.get(name)
+        return int(shape[0]) if shape else None
+
+    def fill(m: dict, key: str, value) -> None:
+        if key not in m and value is not None:
+            m[key] = value
+
+    out = dict(d)
+    if "embed" in shapes and len(shapes["embed"]) == 2:
+        fill(out, "vocab", int(shapes["embed"][0]))
+        fill(out, "width", int(shapes["embed"][1]))
+    layers = d.get("layers")
+    if not isinstance(layers, list):
+        return out
+    out["layers"] = new_layers = []
+    for i, entry in enumerate(layers):
+        if not isinstance(entry, Mapping) or not isinstance(entry.get("mixer"), Mapping):
+            new_layers.append(entry)
+            continue
+        p = f"l{i}.mix."
+        m = dict(entry["mixer"])
+        fill(m, "heads", rows(p + "sink"))
+        H = m.get("heads")
+        if entry.get("type") == "attention" and isinstance(H, int) and H > 0:
+            q, k = rows(p + "q"), rows(p + "k")
+            fill(m, "dim", q // H if q else None)
+            dim = m.get("dim")
+            fill(m, "kv_heads", k // dim if k and isinstance(dim, int) and dim > 0 else None)
+            fill(m, "vdim", dim)
+        elif entry.get("type") == "latent_attention" and isinstance(H, int) and H > 0:
+            fill(m, "q_rank", rows(p + "dq"))
+            fill(m, "kv_rank", rows(p + "dkv.norm"))
+            dkv, uk, uv = rows(p + "dkv"), rows(p + "uk"), rows(p + "uv")
+            if dkv and isinstance(m.get("kv_rank"), int):
+                fill(m, "rot_dim", dkv - m["kv_rank"])
+            fill(m, "dim", uk // H if uk else None)
+            fill(m, "vdim", uv // H if uv else None)
+        e = dict(entry, mixer=m)
+        f = entry.get("mlp")
+        if isinstance(f, Mapping):
+            f = dict(f)
+            expert = dict(f["expert"]) if isinstance(f.get("expert"), Mapping) else {}
+            router = dict(f["router"]) if isinstance(f.get("router"), Mapping) else {}
+            fill(expert, "ff", rows(f"l{i}.mlp.e0.gate"))
+            fill(router, "experts", rows(f"l{i}.mlp.router"))
+            f["expert"], f["router"] = expert, router
+            e["mlp"] = f
+        new_layers.append(e)
+    return out
+
+
 @dataclass(frozen=True)
 class LesaraxConfig:
     vocab: int

@@ -3,7 +3,7 @@ the one decoder class that runs any description."""
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import Any, Callable, Mapping, Tuple
+from typing import Any, Callable, Mapping, Optional, Tuple
 
 from ..config import ConfigError, read_config_json
 from ..parts.spec import ModelSpec
@@ -15,6 +15,9 @@ class Architecture:
     name: str
     read_config: Callable[[Mapping[str, Any]], Any]   # config.json dict -> typed configuration
     describe: Callable[[Any], ModelSpec]               # typed configuration -> ModelSpec
+    # (config.json dict, tensor name -> shape of the stored tensors) -> config.json dict in which the sizes that the
+    # file leaves out are filled in from the shapes; None: the design's config.json names every size
+    sizes_from_tensors: Optional[Callable[[Mapping[str, Any], Mapping[str, Tuple[int, ...]]], Mapping[str, Any]]] = None
 
 
 ARCHITECTURES: Registry = Registry("architecture")
@@ -33,8 +36,13 @@ def architecture_of(config_json: Mapping[str, Any]) -> Architecture:
     raise ConfigError(f"config.json names architecture {candidates!r}; known: {', '.join(ARCHITECTURES.names())}")
 
 
-def describe_model(config_json: Mapping[str, Any]) -> Tuple[Architecture, Any, ModelSpec]:
+def describe_model(config_json: Mapping[str, Any],
+                   tensor_shapes: Optional[Mapping[str, Tuple[int, ...]]] = None) -> Tuple[Architecture, Any, ModelSpec]:
+    """`tensor_shapes` (of a model folder's stored tensors): a design whose config.json may leave sizes to the shapes
+    gets them filled in before the configuration is read."""
     arch = architecture_of(config_json)
+    if tensor_shapes is not None and arch.sizes_from_tensors is not None:
+        config_json = arch.sizes_from_tensors(config_json, tensor_shapes)
     cfg = arch.read_config(config_json)
     spec = arch.describe(cfg)
     spec.validate()

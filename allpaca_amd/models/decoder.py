@@ -15,6 +15,7 @@ from ..parts import CONNECTIONS, EMBEDDINGS, HEADS, NORMS, Block, Runtime, build
 from ..parts.base import CacheNeed
 from ..parts.spec import ModelSpec, ParamSpec
 from ..weights.loader import load_tensors
+from ..weights.safetensors_io import open_model_files
 
 
 class DecoderModel:
@@ -145,8 +146,12 @@ def load_model(model_dir: str, dtype: torch.dtype, device: torch.device | str = 
     chosen by config.json.  `max_positions`: positions the run is set up for (position tables), at most the
     configuration's own limit unless `beyond_configured_positions` (the formulas hold at any position, and the
     reference does not read `max_position_embeddings`; a replay of given tokens may go past it)."""
-    from . import describe_model
-    arch, cfg, spec = describe_model(read_config_json(model_dir))
+    from . import architecture_of, describe_model
+    config_json = read_config_json(model_dir)
+    shapes = None
+    if architecture_of(config_json).sizes_from_tensors is not None:
+        shapes = {n: shape for f in open_model_files(model_dir) for n, (_, shape) in f.entries.items()}
+    arch, cfg, spec = describe_model(config_json, shapes)
     model = DecoderModel(spec)
     tensors = load_tensors(model_dir, model.param_specs(), dtype, spec.forbidden, spec.copies, spec.ignored_suffixes,
                            spec.aliases)

@@ -11,7 +11,7 @@ every pass the stream is mixed with the embedding's output through `loop.in`.  T
 `l<i>.mlp.router`, `l<i>.mlp.e<j>.gate|up|down`, `final.norm`."""
 from __future__ import annotations
 
-from ..config.lesarax import LesaraxAttention, LesaraxConfig
+from ..config.lesarax import LesaraxAttention, LesaraxConfig, sizes_from_tensors
 from ..parts.spec import BlockSpec, ModelSpec, PartSpec, PlanEntry
 from . import ARCHITECTURES, Architecture
 
@@ -59,4 +59,4 @@ def lesarax_spec(cfg: LesaraxConfig) -> ModelSpec:
     )
 
 
-ARCHITECTURES.register("Lesarax", Architecture("lesarax", LesaraxConfig.from_dict, lesarax_spec))
+ARCHITECTURES.register("Lesarax", Architecture("lesarax", LesaraxConfig.from_dict, lesarax_spec, sizes_from_tensors))

@@ -74,8 +74,15 @@ TINY_LE = dict(
     loop=dict(start=0, stop=2, times=4),
     layers=[_layer(_lat(4, 16, 16, 16, 32, 48, 0.18, 10000.0, window=16), _moe(48, 1.0, 3, 1)),
             _layer(_att(2, 1, 32, 0.18, 16, 10000.0), _moe(32, 1.0, 2, 2))])
+# F: a width, heads and latents that are multiples of nothing, one layer alone in the loop, a window of 2
+TINY_LF = dict(
+    architecture="Lesarax", vocab=37, width=50, residual_mult=0.9, norm=dict(eps=1e-6),
+    loop=dict(start=1, stop=2, times=3),
+    layers=[_layer(_att(5, 1, 6, 0.4, 6, 31.0), _moe(7, 0.6, 3, 2)),
+            _layer(_lat(2, 5, 2, 3, 7, 5, 0.45, 13.0, window=2), _moe(9, 1.1, 2, 1))])
 
-CONFIGS = {"LA": (TINY_LA, 31), "LB": (TINY_LB, 32), "LC": (TINY_LC, 33), "LD": (TINY_LD, 34), "LE": (TINY_LE, 35)}
+CONFIGS = {"LA": (TINY_LA, 31), "LB": (TINY_LB, 32), "LC": (TINY_LC, 33), "LD": (TINY_LD, 34), "LE": (TINY_LE, 35),
+           "LF": (TINY_LF, 36)}
 
 
 def planted(cfg: dict, seed: int) -> Dict[str, torch.Tensor]:

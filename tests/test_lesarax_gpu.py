@@ -375,6 +375,24 @@ def test_a_mixer_alone(name):
         close(run_cut(runner, toks, [2, 5, 3]), want, "float32", "portions")
 
 
+def test_a_folder_whose_config_leaves_sizes_to_the_tensors_shapes():
+    import json
+    import shutil
+    from helpers import tmp_root
+    from test_lesarax_plain import bare
+    from allpaca_amd.engine.runner import ModelRunner
+    from allpaca_amd.models import load_model
+    src = model_folder("LA")
+    path = os.path.join(tmp_root(), "LA_bare")
+    shutil.copytree(src, path, dirs_exist_ok=True)
+    with open(os.path.join(path, "config.json"), "w") as f:
+        json.dump(bare(CONFIGS["LA"][0]), f)
+    cfg, model = load_model(path, torch.float32, DEV)
+    assert cfg.vocab == 83 and cfg.layers[0].mixer.q_rank == 20 and cfg.layers[2].mlp.ff == 28
+    toks = tokens_for("LA", 19, 4)
+    close(run_cut(ModelRunner(model, 4, 64, max_requests=2), toks, [19]), oracle_logits(src, toks), "float32", "bare")
+
+
 def test_layers_one_by_one_in_32_bit():
     """The residual after every run of a layer (a looped layer counts each time) against the plain implementation's,
     for a prompt and for its last token alone."""
@@ -393,7 +411,7 @@ def test_layers_one_by_one_in_32_bit():
             close(np.concatenate([got[i], got[n + i]]), want[i], "float32", f"{name} layer run {i}")
 
 
-@pytest.mark.parametrize("name", ["LA", "LB", "LC", "LD", "LE"])
+@pytest.mark.parametrize("name", ["LA", "LB", "LC", "LD", "LE", "LF"])
 @pytest.mark.parametrize("dtype, page_tokens", [("float32", 4), ("bfloat16", 4), ("bfloat16", 16)])
 def test_whole_prompts_decoding_and_portions(name, dtype, page_tokens):
     """(Pages of 16 positions: the bfloat16 run's attention on the matrix-core kernels where they take the sizes; of

@@ -185,3 +185,30 @@ def test_planted_weights_make_the_mechanisms_show():
     assert moved(loose) > 1e-2
     assert moved(dict(cfg, loop=dict(cfg["loop"], times=1))) > 1e-2
     assert moved(other_w={**W, "loop.in": np.concatenate([W["loop.in"][:, :128], 0 * W["loop.in"][:, 128:]], axis=1)}) > 1e-2
+
+
+def bare(cfg):
+    """The configuration without the sizes that the shapes of the tensors give."""
+    import copy
+    out = copy.deepcopy(cfg)
+    out.pop("vocab")
+    out.pop("width")
+    for L in out["layers"]:
+        for k in ("heads", "kv_heads", "dim", "vdim", "q_rank", "kv_rank", "rot_dim"):
+            L["mixer"].pop(k, None)
+        if L["mlp"]:
+            L["mlp"]["expert"].pop("ff")
+            L["mlp"]["router"].pop("experts")
+    return out
+
+
+def test_sizes_that_config_json_leaves_out_come_from_the_tensors_shapes():
+    from allpaca_amd.config import ConfigError
+    from allpaca_amd.config.lesarax import sizes_from_tensors
+    from allpaca_amd.models import describe_model
+    for name, (cfg, _) in CONFIGS.items():
+        shapes = P.tensor_shapes(cfg)
+        assert describe_model(bare(cfg), shapes)[1] == describe_model(cfg)[1], name
+        assert sizes_from_tensors(cfg, shapes) == cfg                 # what the file names stays
+    with pytest.raises(ConfigError, match="vocab"):
+        describe_model(bare(TINY_LA))                                  # no shapes at hand: the sizes are missing
