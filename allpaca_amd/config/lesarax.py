@@ -4,7 +4,8 @@ Keys: `vocab`, `width`, `residual_mult`, `norm.eps`, `loop` ({"start", "stop", "
 `times` times in a row with the same weights; absent or null: every layer once) and `layers`, a list of
 {"type", "mixer", "mlp"}.
   type "attention": `heads`, `kv_heads`, `dim` (query and key size of a head), `vdim` (equal to `dim`: the values are
-      the keys as projected), `scale`, `rot` ({"base", "dims"}: the rotation on a head's first `dims` elements).
+      the keys as projected), `scale`, `rot` ({"base", "dims"}: the rotation on a head's first `dims` elements), `mask`
+      as below (absent: every earlier position).
   type "latent_attention": `heads`, `dim` (unrotated elements of a head's query and key), `rot_dim` (rotated ones),
       `vdim`, `q_rank`, `kv_rank` (sizes of the latents), `scale`, `rot` ({"base", "dims"}, dims = rot_dim), `mask`
       ({"size": n}: a row sees itself and the n - 1 positions before it; absent: every earlier position).
@@ -30,6 +31,7 @@ class LesaraxAttention:
     scale: float
     rot_dims: int
     rot_base: float
+    window: Optional[int] = None
 
 
 @dataclass(frozen=True)
@@ -176,10 +178,12 @@ class LesaraxConfig:
                                   f"(known: 'attention', 'latent_attention')")
             m, mw = _obj(entry, "mixer", where), where + "mixer."
             dims, base = _rot(m, mw)
+            mask = m.get("mask")
+            window = None if mask is None else _int(_obj(m, "mask", mw), "size", mw + "mask.")
             if kind == "attention":
                 mixer = LesaraxAttention(heads=_int(m, "heads", mw), kv_heads=_int(m, "kv_heads", mw),
                                          dim=_int(m, "dim", mw), vdim=_int(m, "vdim", mw), scale=_num(m, "scale", mw),
-                                         rot_dims=dims, rot_base=base)
+                                         rot_dims=dims, rot_base=base, window=window)
                 if mixer.heads % mixer.kv_heads:
                     raise ConfigError(f"config.json: {mw}heads {mixer.heads} is no multiple of kv_heads {mixer.kv_heads}")
                 if mixer.vdim != mixer.dim:
@@ -188,12 +192,10 @@ class LesaraxConfig:
                 if dims > mixer.dim:
                     raise ConfigError(f"config.json: {mw}rot.dims {dims} exceeds dim {mixer.dim}")
             else:
-                mask = m.get("mask")
                 mixer = LesaraxLatent(heads=_int(m, "heads", mw), dim=_int(m, "dim", mw),
                                       rot_dim=_int(m, "rot_dim", mw, least=0), vdim=_int(m, "vdim", mw),
                                       q_rank=_int(m, "q_rank", mw), kv_rank=_int(m, "kv_rank", mw),
-                                      scale=_num(m, "scale", mw), rot_base=base,
-                                      window=None if mask is None else _int(_obj(m, "mask", mw), "size", mw + "mask."))
+                                      scale=_num(m, "scale", mw), rot_base=base, window=window)
                 if dims != mixer.rot_dim:
                     raise ConfigError(f"config.json: {mw}rot.dims {dims} must equal rot_dim {mixer.rot_dim}")
             mlp = entry.get("mlp")

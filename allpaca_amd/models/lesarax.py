@@ -26,7 +26,8 @@ def lesarax_spec(cfg: LesaraxConfig) -> ModelSpec:
         if isinstance(m, LesaraxAttention):
             mixer = PartSpec("sink_attention", dict(
                 hidden_size=D, num_heads=m.heads, num_kv_heads=m.kv_heads, key_dim=m.dim, value_dim=m.vdim,
-                scale=m.scale, rotary_dim=m.rot_dims, rope_theta=m.rot_base, mask="causal", learned_sink=True,
+                scale=m.scale, rotary_dim=m.rot_dims, rope_theta=m.rot_base,
+                mask="causal" if m.window is None else "window", mask_size=m.window or 0, learned_sink=True,
                 values_are_keys=True), "mix.")
         else:
             mixer = PartSpec("latent_attention", dict(

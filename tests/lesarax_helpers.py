@@ -13,9 +13,11 @@ import plain_lesarax as P
 from helpers import tmp_root
 
 
-def _att(heads, kv_heads, dim, scale, rot, base):
-    return dict(type="attention", mixer=dict(heads=heads, kv_heads=kv_heads, dim=dim, vdim=dim, scale=scale,
-                                             rot=dict(base=base, dims=rot)))
+def _att(heads, kv_heads, dim, scale, rot, base, window=None):
+    m = dict(heads=heads, kv_heads=kv_heads, dim=dim, vdim=dim, scale=scale, rot=dict(base=base, dims=rot))
+    if window is not None:
+        m["mask"] = dict(size=window)
+    return dict(type="attention", mixer=m)
 
 
 def _lat(heads, dim, rot_dim, vdim, q_rank, kv_rank, scale, base, window=None):
@@ -74,15 +76,24 @@ TINY_LE = dict(
     loop=dict(start=0, stop=2, times=4),
     layers=[_layer(_lat(4, 16, 16, 16, 32, 48, 0.18, 10000.0, window=16), _moe(48, 1.0, 3, 1)),
             _layer(_att(2, 1, 32, 0.18, 16, 10000.0), _moe(32, 1.0, 2, 2))])
-# F: a width, heads and latents that are multiples of nothing, one layer alone in the loop, a window of 2
+# F: a width, heads and latents that are multiples of nothing, one layer alone in the loop, a window of 2, and a window
+#    on the grouped attention as well
 TINY_LF = dict(
     architecture="Lesarax", vocab=37, width=50, residual_mult=0.9, norm=dict(eps=1e-6),
     loop=dict(start=1, stop=2, times=3),
-    layers=[_layer(_att(5, 1, 6, 0.4, 6, 31.0), _moe(7, 0.6, 3, 2)),
+    layers=[_layer(_att(5, 1, 6, 0.4, 6, 31.0, window=7), _moe(7, 0.6, 3, 2)),
             _layer(_lat(2, 5, 2, 3, 7, 5, 0.45, 13.0, window=2), _moe(9, 1.1, 2, 1))])
+# G: multiples of 8 that are no multiples of 16 or 32 (keys of 80 and 48, values of 40, latents of 72 and 56, experts
+#    72 wide, a window of 50 that is no multiple of a page), 4 of 10 experts
+TINY_LG = dict(
+    architecture="Lesarax", vocab=300, width=192, residual_mult=0.35, norm=dict(eps=1e-6),
+    loop=dict(start=0, stop=2, times=3),
+    layers=[_layer(_lat(6, 48, 32, 40, 72, 56, 0.11, 10000.0, window=50), _moe(72, 1.0, 10, 4)),
+            _layer(_att(8, 4, 48, 0.14, 32, 20000.0), _moe(72, 1.0, 10, 4)),
+            _layer(_lat(3, 24, 8, 24, 40, 24, 0.17, 10000.0, window=23), None)])
 
 CONFIGS = {"LA": (TINY_LA, 31), "LB": (TINY_LB, 32), "LC": (TINY_LC, 33), "LD": (TINY_LD, 34), "LE": (TINY_LE, 35),
-           "LF": (TINY_LF, 36)}
+           "LF": (TINY_LF, 36), "LG": (TINY_LG, 37)}
 
 
 def planted(cfg: dict, seed: int) -> Dict[str, torch.Tensor]:

@@ -103,7 +103,7 @@ def experts(h: np.ndarray, W: Dict[str, np.ndarray], p: str, n_experts: int, top
 
 # ---------------------------------------------------------------------------------------------- the two mixers
 def attention_mixer(h: np.ndarray, W: Dict[str, np.ndarray], p: str, m: dict, rnd: Callable = exact) -> np.ndarray:
-    """Grouped heads whose values are the keys as projected (before the rotation)."""
+    """Grouped heads whose values are the keys as projected (before the rotation); a window if the mixer names one."""
     T = h.shape[0]
     H, G, dk = m["heads"], m["kv_heads"], m["dim"]
     pos = np.arange(T)
@@ -111,7 +111,7 @@ def attention_mixer(h: np.ndarray, W: Dict[str, np.ndarray], p: str, m: dict, rn
     k = rnd(h @ W[p + "k"].T).reshape(T, G, dk)
     r, base = m["rot"]["dims"], m["rot"]["base"]
     o = sink_attention(rnd(rotate_front(q, pos, base, r)), rnd(rotate_front(k, pos, base, r)), k, m["scale"],
-                       W[p + "sink"])
+                       W[p + "sink"], window=(m.get("mask") or {}).get("size"))
     return rnd(o.reshape(T, -1)) @ W[p + "o"].T
 
 
