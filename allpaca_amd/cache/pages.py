@@ -21,6 +21,7 @@ import ctypes
 from dataclasses import dataclass
 from typing import Dict, Hashable, List, Optional, Sequence, Tuple
 
+from ..kernels.host import MAX_PAGED_GROUPS
 from ..parts.base import CacheNeed, need_kind
 
 FREED = -1  # block-table entry of a page that a window has passed
@@ -181,8 +182,8 @@ class CacheManager:
             num_pages = [num_pages] * len(paged)
         if len(num_pages) != len(paged):
             raise ValueError(f"{len(paged)} paged groups but {len(num_pages)} pool sizes")
-        if len(paged) > 8:
-            raise ValueError(f"{len(paged)} paged groups: the cache manager keeps books for at most 8")
+        if len(paged) > MAX_PAGED_GROUPS:
+            raise ValueError(f"{len(paged)} paged groups: the cache manager keeps books for at most {MAX_PAGED_GROUPS}")
         if any(n <= 0 for n in num_pages) or max_requests <= 0:
             raise ValueError("a page pool needs at least one page")
         self._lib = L = _host()
@@ -199,7 +200,7 @@ class CacheManager:
         self.max_requests = max_requests
         self._ids: Dict[Hashable, int] = {}
         self._next_id = 0
-        self._need = (ctypes.c_int * 8)()
+        self._need = (ctypes.c_int * MAX_PAGED_GROUPS)()
         self._table = (ctypes.c_int * 64)()
         # plan entry -> ("paged", group index, index inside the group) | ("state", ...) ; filled for owners only
         self.location: Dict[int, Tuple[str, int, int]] = {}

@@ -6,7 +6,6 @@
 #include <unordered_map>
 #include <vector>
 
-#define APC_MAX_GROUPS 8
 #define APC_PAGE_FREED (-1)           // block-table entry of a page that a window has passed
 
 #define APC_CACHE_ALREADY_LIVE (-20)

@@ -9,6 +9,8 @@
 #include <stddef.h>
 #include <stdint.h>
 
+#define APC_MAX_GROUPS 16            // paged groups a model may have (kernels/host.py: MAX_PAGED_GROUPS)
+
 #define APC_HOST_EXPORT extern "C" __attribute__((visibility("default")))
 
 // error codes beside the kernels' own (-1 bad argument, -2 unsupported)
@@ -63,8 +65,8 @@ struct ApcStep {
   const int* tile_row0;
   const int* tile_rows;
   int n_groups;
-  const int* table[8];        // per paged group: [S][table_width]
-  int table_width[8];
+  const int* table[APC_MAX_GROUPS];        // per paged group: [S][table_width]
+  int table_width[APC_MAX_GROUPS];
   int max_decode_context;     // largest position + 1 among the single-row segments
   int all_rows_decode;        // every row is a single-row segment (decode_rows is then not read)
   int max_prompt_keys;        // largest position + rows among the longer segments (how attention cuts their keys)

@@ -26,6 +26,8 @@ class ApcPlanEntry(Structure):
                 ("writes", c_int)]
 
 
+MAX_PAGED_GROUPS = 16      # csrc/host/host.h: APC_MAX_GROUPS
+
 STEP_ARRAYS = ("tokens", "positions", "row_seg", "seg_row0", "seg_rows", "seg_pos0", "state_slots", "logit_rows",
                "decode_rows", "tile_row0", "tile_rows")
 
@@ -33,7 +35,7 @@ STEP_ARRAYS = ("tokens", "positions", "row_seg", "seg_row0", "seg_rows", "seg_po
 class ApcStep(Structure):
     _fields_ = ([("T", c_int), ("S", c_int), ("R", c_int), ("n_decode", c_int), ("n_tiles", c_int)]
                 + [(name, c_void_p) for name in STEP_ARRAYS]
-                + [("n_groups", c_int), ("table", c_void_p * 8), ("table_width", c_int * 8),
+                + [("n_groups", c_int), ("table", c_void_p * MAX_PAGED_GROUPS), ("table_width", c_int * MAX_PAGED_GROUPS),
                    ("max_decode_context", c_int), ("all_rows_decode", c_int), ("max_prompt_keys", c_int)])
 
 
@@ -43,7 +45,8 @@ class ApcStepFinding(Structure):
 
 class ApcPacked(Structure):
     _fields_ = [("T", c_int), ("S", c_int), ("R", c_int), ("n_decode", c_int), ("n_tiles", c_int), ("total", c_int),
-                ("off", c_int * 11), ("n_groups", c_int), ("table_off", c_int * 8), ("table_width", c_int * 8),
+                ("off", c_int * 11), ("n_groups", c_int), ("table_off", c_int * MAX_PAGED_GROUPS),
+                ("table_width", c_int * MAX_PAGED_GROUPS),
                 ("max_decode_context", c_int), ("max_prompt_keys", c_int), ("max_context", c_int), ("max_rows", c_int)]
 
 

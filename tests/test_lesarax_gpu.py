@@ -394,6 +394,26 @@ def test_a_folder_whose_config_leaves_sizes_to_the_tensors_shapes():
     close(run_cut(ModelRunner(model, 4, 64, max_requests=2), toks, [19]), oracle_logits(src, toks), "float32", "bare")
 
 
+def test_ten_layers_with_ten_different_windows():
+    """Every layer's pages are a group of their own (ten block tables a request), and every window gives pages back at
+    its own pace."""
+    from helpers import tmp_root
+    cfg = dict(architecture="Lesarax", vocab=30, width=16, residual_mult=0.5, norm=dict(eps=1e-5),
+               loop=dict(start=2, stop=5, times=2),
+               layers=[_layer(_lat(2, 4, 4, 4, 8, 6, 0.4, 50.0, window=2 + 3 * i), None) for i in range(10)])
+    path = write_folder(os.path.join(tmp_root(), "lesarax_windows"), cfg, 44)
+    from allpaca_amd.engine.runner import ModelRunner
+    from allpaca_amd.models import load_model
+    _, model = load_model(path, torch.float32, DEV)
+    runner = ModelRunner(model, 4, 24, max_requests=2, poison_free_pages=True)
+    assert len(runner.cache.paged_groups) == 10
+    toks = np.random.default_rng(6).integers(0, 30, size=60).tolist()
+    want = P.forward(*P.read_model_folder(path), toks)
+    close(run_cut(runner, toks, [60]), want, "float32", "whole")
+    close(run_cut(runner, toks, [7, 1, 1, 30, 2, 1]), want, "float32", "portions")
+    runner.cache.check()
+
+
 def test_layers_one_by_one_in_32_bit():
     """The residual after every run of a layer (a looped layer counts each time) against the plain implementation's,
     for a prompt and for its last token alone."""
