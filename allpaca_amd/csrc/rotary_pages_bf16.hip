@@ -6,7 +6,9 @@
 // range is handled together with its partner, the piece rot/2 elements further on (rot/2 is a multiple of 8, so the
 // partners of a piece's elements are a piece): the thread reads both, turns the 8 pairs and writes both, so q may be
 // rotated where it lies; the thread of a piece in the second half does nothing.  A key's piece goes into the page
-// as one 16-byte store; a value's 8 elements go to 8 rows of the transposed value block, slot by slot.
+// as one 16-byte store; a value's 8 elements go to 8 rows of the transposed value block, slot by slot.  In steps of
+// many rows the values go through rotary_pages_values_kernel instead (16 rows x 128 columns through LDS, 8 slots of a
+// column in one store).
 // The second part of a key (the part all heads share, or a head's own) may be float32 rows.
 #include "mfma.h"
 #include <math.h>
@@ -41,10 +43,10 @@ __global__ __launch_bounds__(256) void rotary_pages_bf16_kernel(
     const bf16_t* __restrict__ ka, int ldka, int ka_off, int da, const void* __restrict__ kb, int kb_f32, int ldkb,
     int kb_off, int db, int kb_shared, int k_rot0, const bf16_t* __restrict__ v, int ldv, int v_off, int dv, int G,
     int rot, const float* __restrict__ cos_sin, const int* __restrict__ positions, const int* __restrict__ row_seg,
-    const int* __restrict__ block_table, int max_blocks, bf16_t* __restrict__ cache, int P) {
+    const int* __restrict__ block_table, int max_blocks, bf16_t* __restrict__ cache, int P, int with_values) {
   const int r = blockIdx.x;
   const int dk = da + db, half = rot / 2;
-  const int nq = H * (dq / 8), nk = G * (dk / 8), nv = G * (dv / 8);
+  const int nq = H * (dq / 8), nk = G * (dk / 8), nv = with_values ? G * (dv / 8) : 0;
   const int item = blockIdx.y * 256 + threadIdx.x;
   if (item >= nq + nk + nv) return;
   const int pos = positions[r];
@@ -106,6 +108,61 @@ __global__ __launch_bounds__(256) void rotary_pages_bf16_kernel(
   }
 }
 
+// The values of 16 rows x 128 columns (kv head * dv + element) through LDS into the transposed value blocks: where 8
+// rows are 8 consecutive slots of one page that start at a multiple of 8, a column's 8 values leave as one 16-byte
+// store; else slot by slot.
+constexpr int VR = 16, VC = 128, VPAD = 8;
+
+__global__ __launch_bounds__(256) void rotary_pages_values_kernel(
+    const bf16_t* __restrict__ v, int ldv, int v_off, int dk, int dv, int G, const int* __restrict__ positions,
+    const int* __restrict__ row_seg, const int* __restrict__ block_table, int max_blocks, bf16_t* __restrict__ cache,
+    int P, int n_rows) {
+  __shared__ __attribute__((aligned(16))) bf16_t vt[VR][VC + VPAD];
+  __shared__ long long base_s[VR];      // element offset of the row's page; -1: no such row
+  __shared__ int slot_s[VR];
+  const int tid = threadIdx.x, r0 = blockIdx.x * VR, c0 = blockIdx.y * VC;
+  if (tid < VR) {
+    const int t = r0 + tid;
+    long long base = -1;
+    int slot = 0;
+    if (t < n_rows) {
+      const int pos = positions[t];
+      base = (long long)block_table[(size_t)row_seg[t] * max_blocks + pos / P] * G * P * (dk + dv);
+      slot = pos % P;
+    }
+    base_s[tid] = base;
+    slot_s[tid] = slot;
+  }
+  __syncthreads();
+  const int h = tid % 2;                // the half (8 rows) whose columns this thread stores
+  bool run = P % 8 == 0 && slot_s[8 * h] % 8 == 0;
+#pragma unroll
+  for (int r = 0; r < 8; ++r)
+    run = run && base_s[8 * h + r] >= 0 && base_s[8 * h + r] == base_s[8 * h] && slot_s[8 * h + r] == slot_s[8 * h] + r;
+  const int cw = min(VC, G * dv - c0), pieces = cw / 8;
+  for (int item = tid; item < VR * pieces; item += 256) {
+    const int r = item / pieces, p = item % pieces;
+    if (r0 + r < n_rows)
+      *reinterpret_cast<Frag*>(&vt[r][p * 8]) = load_frag(v + (size_t)(r0 + r) * ldv + v_off + c0 + p * 8);
+  }
+  __syncthreads();
+  for (int item = tid; item < 2 * cw; item += 256) {      // item % 2 == h: 256 is even
+    const int col = c0 + item / 2, g = col / dv, e = col % dv;
+    const size_t at = ((size_t)g * (dk + dv) + dk + e) * P;   // the column's row of slots inside a page
+    if (run) {
+      Frag f;
+#pragma unroll
+      for (int w = 0; w < 4; ++w)
+        f.w[w] = (uint32_t)vt[8 * h + 2 * w][item / 2] | ((uint32_t)vt[8 * h + 2 * w + 1][item / 2] << 16);
+      *reinterpret_cast<Frag*>(cache + base_s[8 * h] + at + slot_s[8 * h]) = f;
+    } else {
+#pragma unroll
+      for (int r = 0; r < 8; ++r)
+        if (base_s[8 * h + r] >= 0) cache[base_s[8 * h + r] + at + slot_s[8 * h + r]] = vt[8 * h + r][item / 2];
+    }
+  }
+}
+
 bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
 
 }  // namespace
@@ -134,12 +191,21 @@ APC_EXPORT int apc_rotary_pages_bf16(const void* q, int ldq, int q_off, int H, i
       !aligned16(q) || !aligned16(q_out) || !aligned16(ka) || !aligned16(v) || (db && !aligned16(kb)) ||
       !aligned16(cache) || (rot && !aligned16(cos_sin)))
     return APC_ERR_UNSUPPORTED;
-  const long items = (long)H * (dq / 8) + (long)G * ((da + db) / 8) + (long)G * (dv / 8);
+  // Steps of many rows (prompt portions): the values go through a kernel of their own that gathers 8 slots of a
+  // column into one store.  Both ways write the same bits.
+  const bool apart = n_rows >= 2 * VR && page_tokens % 8 == 0 && ((long)G * dv + VC - 1) / VC <= 65535;
+  const long items = (long)H * (dq / 8) + (long)G * ((da + db) / 8) + (apart ? 0 : (long)G * (dv / 8));
   if (items > 65535L * 256) return APC_ERR_UNSUPPORTED;
+  if (apart) {
+    hipLaunchKernelGGL(rotary_pages_values_kernel, dim3((n_rows + VR - 1) / VR, (unsigned)((G * dv + VC - 1) / VC)),
+                       dim3(256), 0, stream, (const bf16_t*)v, ldv, v_off, da + db, dv, G, positions, row_seg,
+                       block_table, max_blocks, (bf16_t*)cache, page_tokens, n_rows);
+    APC_LAUNCH_CHECK();
+  }
   hipLaunchKernelGGL(rotary_pages_bf16_kernel, dim3(n_rows, (unsigned)((items + 255) / 256)), dim3(256), 0, stream,
                      (const bf16_t*)q, ldq, q_off, H, dq, q_rot0, (bf16_t*)q_out, ldqo, (const bf16_t*)ka, ldka, ka_off,
                      da, kb, kb_f32, ldkb, kb_off, db, kb_shared, k_rot0, (const bf16_t*)v, ldv, v_off, dv, G, rot,
-                     cos_sin, positions, row_seg, block_table, max_blocks, (bf16_t*)cache, page_tokens);
+                     cos_sin, positions, row_seg, block_table, max_blocks, (bf16_t*)cache, page_tokens, apart ? 0 : 1);
   APC_LAUNCH_CHECK();
   return 0;
 }

@@ -154,7 +154,7 @@ def test_keys_put_together_from_a_head_s_own_part_and_a_rotated_part_all_heads_s
     rng = np.random.default_rng(H * dn + dr)
     tdt = DTYPES[dtype]
     dk = dn + dr
-    segs, lens = [(2 * P_ - 1, P_ + 2), (7, 1)], [3 * P_ + 1, 8]
+    segs, lens = [(2 * P_ - 1, 3 * P_ + 2), (7, 1)], [5 * P_ + 1, 8]
     n_pages, tables = scattered_tables(rng, lens, P_)
     T = sum(n for _, n in segs)
     q = bf(rng.normal(size=(T, H, dk)))
@@ -165,7 +165,7 @@ def test_keys_put_together_from_a_head_s_own_part_and_a_rotated_part_all_heads_s
     cache = torch.full((n_pages + 1, H, P_ * (dk + dv)), float("nan"), dtype=tdt, device=DEV)
     step = make_step(segs, tables)
     base = 900.0
-    table = rotary_table(dr, base, Runtime(torch.device(DEV), tdt, 4 * P_))
+    table = rotary_table(dr, base, Runtime(torch.device(DEV), tdt, 6 * P_))
     ops.rotary_pages(q_dev, 0, H, dk, dn, q_dev, dev(kv, tdt), 0, dn, dev(a), off, dr, True, dn, dev(kv, tdt), H * dn, dv,
                      H, dr, table, step, step.block_tables[0], cache, P_)
     got_q, got_pages = q_dev.float().cpu().numpy().reshape(T, H, dk), cache.float().cpu().numpy()
