@@ -461,6 +461,70 @@ __global__ __launch_bounds__(NT) void streams_step_f4_kernel(float* __restrict__
   }
 }
 
+// One stream (S = 1) with a sublayer's output to add: x <- mix x + out_w y, h = rms_norm(in_w x) * norm_w.  The same
+// arithmetic in the same order as the kernel above; every load of the row is issued before the first store, so a
+// thread waits for memory once and not once a piece.
+template <int NT, int VPT>
+__global__ __launch_bounds__(NT) void stream_add_f4_kernel(float* __restrict__ x, int D, const void* __restrict__ y,
+                                                           int y_dtype, int ldy, const float* __restrict__ mix,
+                                                           const float* __restrict__ out_w,
+                                                           const float* __restrict__ in_w,
+                                                           const float* __restrict__ norm_w, float eps,
+                                                           void* __restrict__ h, int h_dtype, int ldh) {
+  __shared__ float red[NT / WAVE];
+  const int r = blockIdx.x, n4 = D / 4;
+  float4* xr = reinterpret_cast<float4*>(x + (size_t)r * D);
+  const float m = mix[0], o = out_w[0], wi = in_w ? in_w[0] : 0.f;
+  float4 v[VPT], yy[VPT];
+#pragma unroll
+  for (int k = 0; k < VPT; ++k) {
+    const int i = threadIdx.x + k * NT;
+    v[k] = yy[k] = float4{0.f, 0.f, 0.f, 0.f};
+    if (i >= n4) continue;
+    v[k] = xr[i];
+    if (y_dtype == APC_F32) {
+      yy[k] = reinterpret_cast<const float4*>((const float*)y + (size_t)r * ldy)[i];
+    } else {
+      const uint2 p = reinterpret_cast<const uint2*>((const bf16_t*)y + (size_t)r * ldy)[i];
+      yy[k] = float4{__uint_as_float(p.x << 16), __uint_as_float(p.x & 0xffff0000u), __uint_as_float(p.y << 16),
+                     __uint_as_float(p.y & 0xffff0000u)};
+    }
+  }
+  float ss = 0.f;
+#pragma unroll
+  for (int k = 0; k < VPT; ++k) {
+    const int i = threadIdx.x + k * NT;
+    if (i >= n4) continue;
+    float4 a = float4{fmaf(m, v[k].x, 0.f), fmaf(m, v[k].y, 0.f), fmaf(m, v[k].z, 0.f), fmaf(m, v[k].w, 0.f)};
+    a = float4{fmaf(o, yy[k].x, a.x), fmaf(o, yy[k].y, a.y), fmaf(o, yy[k].z, a.z), fmaf(o, yy[k].w, a.w)};
+    xr[i] = a;
+    if (in_w) {
+      a = float4{fmaf(wi, a.x, 0.f), fmaf(wi, a.y, 0.f), fmaf(wi, a.z, 0.f), fmaf(wi, a.w, 0.f)};
+      ss = fmaf(a.x, a.x, ss); ss = fmaf(a.y, a.y, ss); ss = fmaf(a.z, a.z, ss); ss = fmaf(a.w, a.w, ss);
+    }
+    v[k] = a;
+  }
+  if (!in_w) return;
+  ss = block_sum<NT>(ss, red);
+  const float inv = 1.0f / sqrtf(ss / (float)D + eps);
+#pragma unroll
+  for (int k = 0; k < VPT; ++k) {
+    const int i = threadIdx.x + k * NT;
+    if (i >= n4) continue;
+    float4 g = float4{1.f, 1.f, 1.f, 1.f};
+    if (norm_w) g = reinterpret_cast<const float4*>(norm_w)[i];
+    const float4 u = float4{(v[k].x * inv) * g.x, (v[k].y * inv) * g.y, (v[k].z * inv) * g.z, (v[k].w * inv) * g.w};
+    if (h_dtype == APC_F32) {
+      reinterpret_cast<float4*>((float*)h + (size_t)r * ldh)[i] = u;
+    } else {
+      uint2 p;
+      p.x = pack_bf16x2(u.x, u.y);
+      p.y = pack_bf16x2(u.z, u.w);
+      reinterpret_cast<uint2*>((bf16_t*)h + (size_t)r * ldh)[i] = p;
+    }
+  }
+}
+
 APC_EXPORT int apc_streams_step(float* x, int n_rows, int S, int D, const void* y, int y_dtype, int ldy,
                                 const float* mix, const float* out_w, const float* in_w, const float* norm_w, float eps,
                                 void* h, int h_dtype, int ldh, const int* rows, hipStream_t stream) {
@@ -471,6 +535,18 @@ APC_EXPORT int apc_streams_step(float* x, int n_rows, int S, int D, const void* 
   if (S > MAX_STREAMS) return APC_ERR_UNSUPPORTED;
   const bool wide = D % 4 == 0 && D <= 256 * 4 * 8 && !((uintptr_t)x & 15u) && !((uintptr_t)norm_w & 15u) &&
                     (!y || (ldy % 4 == 0 && !((uintptr_t)y & 15u))) && (!in_w || (ldh % 4 == 0 && !((uintptr_t)h & 15u)));
+  if (wide && S == 1 && y && !rows) {
+#define SA_LAUNCH(VPT_)                                                                                           \
+  hipLaunchKernelGGL((stream_add_f4_kernel<256, VPT_>), dim3(n_rows), dim3(256), 0, stream, x, D, y, y_dtype, ldy, \
+                     mix, out_w, in_w, norm_w, eps, h, h_dtype, ldh)
+    if (D <= 1024) SA_LAUNCH(1);
+    else if (D <= 2048) SA_LAUNCH(2);
+    else if (D <= 4096) SA_LAUNCH(4);
+    else SA_LAUNCH(8);
+#undef SA_LAUNCH
+    APC_LAUNCH_CHECK();
+    return 0;
+  }
   if (wide) {
 #define ST_LAUNCH(VPT_)                                                                                              \
   hipLaunchKernelGGL((streams_step_f4_kernel<256, VPT_>), dim3(n_rows), dim3(256), 0, stream, x, S, D, y, y_dtype, ldy, \
