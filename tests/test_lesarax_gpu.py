@@ -188,7 +188,8 @@ def test_keys_put_together_from_a_head_s_own_part_and_a_rotated_part_all_heads_s
 @pytest.mark.parametrize("H, G, dk, dv, P_, W", [(4, 2, 12, 12, 4, 0), (3, 3, 16, 14, 3, 37), (10, 2, 64, 64, 16, 0),
                                                  (4, 4, 48, 32, 16, 88), (4, 4, 32, 64, 8, 64), (2, 1, 128, 128, 16, 100),
                                                  (16, 2, 64, 64, 16, 0), (5, 5, 80, 40, 16, 50), (6, 3, 24, 24, 16, 0),
-                                                 (2, 2, 200, 72, 16, 130)])
+                                                 (2, 2, 200, 72, 16, 130), (12, 4, 96, 96, 16, 0), (7, 7, 160, 96, 16, 200),
+                                                 (4, 1, 256, 256, 16, 0)])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_sink_window_and_head_gate_over_pages_with_one_key_that_stands_out(H, G, dk, dv, P_, W, dtype):
     """Attention with a learned sink a head, a window (W > 0) or none, and a gate a head, on scattered pages whose
