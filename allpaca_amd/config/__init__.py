@@ -11,6 +11,7 @@ from .llama import ConfigError, Llama3RopeScaling, LlamaConfig
 from .gulidra import GulidraConfig
 from .lesarax import LesaraxConfig
 from .risizen import RisizenConfig
+from .seredra import SeredraConfig
 
 
 def read_config_json(model_dir: str) -> dict:
@@ -27,7 +28,7 @@ def read_config_json(model_dir: str) -> dict:
     return d
 
 
-__all__ = ["ConfigError", "EngineConfig", "GulidraConfig", "LesaraxConfig", "Llama3RopeScaling", "LlamaConfig", "RisizenConfig", "read_config_json"]
+__all__ = ["ConfigError", "EngineConfig", "GulidraConfig", "LesaraxConfig", "Llama3RopeScaling", "LlamaConfig", "RisizenConfig", "SeredraConfig", "read_config_json"]
 
 
 def preset(name: str) -> dict:

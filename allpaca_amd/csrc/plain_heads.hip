@@ -15,6 +15,8 @@ constexpr int MAX_HEAD = 1024;
 //   key of kv head g, dk = da + db elements: first ka[t][ka_off + g * da + i] (i < da), then
 //       kb[t][kb_off + (kb_shared ? 0 : g * db) + i] (i < db); elements [k_rot0, k_rot0 + rot) of the whole are rotated
 //   value of kv head g: v[t][v_off + g * dv + e], as it is
+// With `q_norm_w` [dq] (`k_norm_w` [da + db]) a query (key) head is first divided by its root mean square over the
+// head, sqrt(mean(x^2) + eps), and multiplied with the weights, which all heads share; values are never normed.
 // The rotation pairs element i with element i + rot/2 of the range: (x, y) -> (x c - y s, y c + x s), c and s from
 // cos_sin[position][2][rot/2].
 // pages: page = block_table[seg][pos / P]; keys page[g][slot * dk + i], values page[g][P * dk + e * P + slot], a page
@@ -25,7 +27,8 @@ __global__ __launch_bounds__(64) void rotary_pages_kernel(
     const void* __restrict__ kb, int kb_dtype, int ldkb, int kb_off, int db, int kb_shared, int k_rot0,
     const void* __restrict__ v, int v_dtype, int ldv, int v_off, int dv, int G, int rot,
     const float* __restrict__ cos_sin, const int* __restrict__ positions, const int* __restrict__ row_seg,
-    const int* __restrict__ block_table, int max_blocks, void* __restrict__ cache, int cache_dtype, int P) {
+    const int* __restrict__ block_table, int max_blocks, void* __restrict__ cache, int cache_dtype, int P,
+    const float* __restrict__ q_norm_w, const float* __restrict__ k_norm_w, float eps) {
   __shared__ float xs[MAX_HEAD];
   const int r = blockIdx.x, hh = blockIdx.y, lane = threadIdx.x;
   const int pos = positions[r];
@@ -43,6 +46,14 @@ __global__ __launch_bounds__(64) void rotary_pages_kernel(
     xs[i] = x;
   }
   __syncthreads();
+  const float* nw = is_q ? q_norm_w : k_norm_w;
+  if (nw) {
+    float ss = 0.f;
+    for (int i = lane; i < d; i += WAVE) ss = fmaf(xs[i], xs[i], ss);
+    const float inv = 1.0f / sqrtf(wave_sum(ss) / (float)d + eps);
+    for (int i = lane; i < d; i += WAVE) xs[i] = (xs[i] * inv) * nw[i];      // (a lane's own elements)
+    __syncthreads();
+  }
   size_t key_base = 0, val_base = 0;
   if (!is_q) {
     const int dk = da + db;
@@ -78,7 +89,7 @@ APC_EXPORT int apc_rotary_pages(const void* q, int q_dtype, int ldq, int q_off, 
                                 const void* v, int v_dtype, int ldv, int v_off, int dv, int G, int rot,
                                 const float* cos_sin, const int* positions, const int* row_seg, const int* block_table,
                                 int max_blocks, void* cache, int cache_dtype, int page_tokens, int n_rows,
-                                hipStream_t stream) {
+                                const float* q_norm_w, const float* k_norm_w, float eps, hipStream_t stream) {
   if (n_rows <= 0) return 0;
   if (H < 0 || G < 0 || H + G <= 0 || rot < 0 || rot % 2 || (rot && !cos_sin) || !positions) return APC_ERR_BAD_ARG;
   if (H && (!q || !q_out || dq <= 0 || q_rot0 < 0 || q_rot0 + rot > dq || ldqo < H * dq)) return APC_ERR_BAD_ARG;
@@ -89,7 +100,7 @@ APC_EXPORT int apc_rotary_pages(const void* q, int q_dtype, int ldq, int q_off, 
   hipLaunchKernelGGL(rotary_pages_kernel, dim3(n_rows, H + G), dim3(64), 0, stream, q, q_dtype, ldq, q_off, H, dq,
                      q_rot0, q_out, qo_dtype, ldqo, ka, ka_dtype, ldka, ka_off, da, kb, kb_dtype, ldkb, kb_off, db,
                      kb_shared, k_rot0, v, v_dtype, ldv, v_off, dv, G, rot, cos_sin, positions, row_seg, block_table,
-                     max_blocks, cache, cache_dtype, page_tokens);
+                     max_blocks, cache, cache_dtype, page_tokens, q_norm_w, k_norm_w, eps);
   APC_LAUNCH_CHECK();
   return 0;
 }

@@ -21,7 +21,10 @@ constexpr int MAX_STREAMS = 16;
 // u of the n-1 positions ahead of a segment's first row comes from state[slot][n-1][width] (zero for a new request:
 // the sequence starts with zeros).  `conv_state_kernel` moves the state on afterwards.
 //   q, k:  y / sqrt(mean(y^2) + eps)  if `unit_norm`, the mean over the head, or over each piece of `norm_dim`
-//          elements of it (norm_dim divides dk; 0: the whole head); times q_norm_w / k_norm_w [norm_dim] if given
+//          elements of it (norm_dim divides dk; 0: the whole head); times q_norm_w / k_norm_w [norm_dim] if given.
+//          `norm_rows`: the mean is taken over all heads of q (of k) at once and the weights are [H * dk] ([G * dk]);
+//          every wave forms the sum over the whole projection for itself, in one order
+//   q:     times 1 + qt_coef * ln(floor((pos + 1) / qt_every) + 1) at position pos, if qt_every > 0
 // pages: page = block_table[seg][pos / P]; keys page[g][slot * dk + i], values page[g][P * dk + e * P + slot]
 // (a key's elements lie together, a value element's slots lie together), a page being G * P * (dk + dv) elements.
 // ---------------------------------------------------------------------------
@@ -30,8 +33,9 @@ __global__ __launch_bounds__(64) void conv_heads_kernel(
     const float* __restrict__ bias, const float* __restrict__ conv_w, int taps, const float* __restrict__ state,
     int width, const int* __restrict__ row_seg, const int* __restrict__ seg_row0, const int* __restrict__ slots,
     const int* __restrict__ positions, int unit_norm, float eps, int norm_dim, const float* __restrict__ q_norm_w,
-    const float* __restrict__ k_norm_w, void* __restrict__ q_out, int q_dtype, int ldq,
-    const int* __restrict__ block_table, int max_blocks, void* __restrict__ cache, int cache_dtype, int P) {
+    const float* __restrict__ k_norm_w, int norm_rows, float qt_coef, int qt_every, void* __restrict__ q_out,
+    int q_dtype, int ldq, const int* __restrict__ block_table, int max_blocks, void* __restrict__ cache,
+    int cache_dtype, int P) {
   const int r = blockIdx.x, hh = blockIdx.y, lane = threadIdx.x;
   int kind, head, d, col0;
   if (hh < H) { kind = 0; head = hh; d = dk; col0 = q_off + head * dk; }
@@ -41,6 +45,18 @@ __global__ __launch_bounds__(64) void conv_heads_kernel(
   const int i_in_seg = r - seg_row0[seg];
   const float* st = (taps > 1) ? state + (size_t)slots[seg] * (taps - 1) * width : nullptr;
 
+  auto channel = [&](int c) -> float {         // the convolution's output of column c of this row
+    const float b = bias ? bias[c] : 0.f;
+    if (!conv_w) return load_f(proj, in_dtype, (size_t)r * ld + c) + b;
+    float acc = 0.f;
+    for (int j = 0; j < taps; ++j) {            // oldest first: the order of the sum is that of the taps
+      const int back = taps - 1 - j;
+      const float u = back <= i_in_seg ? load_f(proj, in_dtype, (size_t)(r - back) * ld + c) + b
+                                       : st[(size_t)(taps - 1 - (back - i_in_seg)) * width + c];
+      acc = fmaf(conv_w[(size_t)c * taps + j], u, acc);
+    }
+    return acc;
+  };
   float y[MAX_PER_LANE];
   float ss = 0.f;
 #pragma unroll
@@ -48,25 +64,26 @@ __global__ __launch_bounds__(64) void conv_heads_kernel(
     const int i = lane + e * WAVE;
     y[e] = 0.f;
     if (i < d) {
-      const int c = col0 + i;
-      const float b = bias ? bias[c] : 0.f;
-      float acc;
-      if (conv_w) {
-        acc = 0.f;
-        for (int j = 0; j < taps; ++j) {          // oldest first: the order of the sum is that of the taps
-          const int back = taps - 1 - j;
-          const float u = back <= i_in_seg ? load_f(proj, in_dtype, (size_t)(r - back) * ld + c) + b
-                                           : st[(size_t)(taps - 1 - (back - i_in_seg)) * width + c];
-          acc = fmaf(conv_w[(size_t)c * taps + j], u, acc);
-        }
-      } else {
-        acc = load_f(proj, in_dtype, (size_t)r * ld + c) + b;
-      }
-      y[e] = acc;
-      ss = fmaf(acc, acc, ss);
+      y[e] = channel(col0 + i);
+      ss = fmaf(y[e], y[e], ss);
     }
   }
-  if (unit_norm && kind != 2) {
+  if (unit_norm && kind != 2 && norm_rows) {
+    const int n = (kind == 0 ? H : G) * dk, c0 = kind == 0 ? q_off : k_off;
+    float tot = 0.f;
+    for (int i = lane; i < n; i += WAVE) {
+      const float v = channel(c0 + i);
+      tot = fmaf(v, v, tot);
+    }
+    const float inv = 1.0f / sqrtf(wave_sum(tot) / (float)n + eps);
+    const float* nw = kind == 0 ? q_norm_w : k_norm_w;
+#pragma unroll
+    for (int e = 0; e < MAX_PER_LANE; ++e) {
+      const int i = lane + e * WAVE;
+      y[e] = y[e] * inv;
+      if (nw && i < d) y[e] *= nw[(size_t)head * dk + i];
+    }
+  } else if (unit_norm && kind != 2) {
     const int nd = norm_dim > 0 ? norm_dim : d;
     const float* nw = kind == 0 ? q_norm_w : k_norm_w;
     if (nd == d) {
@@ -103,7 +120,8 @@ __global__ __launch_bounds__(64) void conv_heads_kernel(
       }
     }
   }
-  const float inv = 1.f;
+  const int pos = positions[r];
+  const float inv = (kind == 0 && qt_every > 0) ? 1.0f + qt_coef * logf((float)((pos + 1) / qt_every) + 1.0f) : 1.f;
 
   if (kind == 0) {
 #pragma unroll
@@ -113,7 +131,6 @@ __global__ __launch_bounds__(64) void conv_heads_kernel(
     }
     return;
   }
-  const int pos = positions[r];
   const int page = block_table[(size_t)seg * max_blocks + pos / P];
   const size_t base = ((size_t)page * G + head) * (size_t)P * (dk + dv);
 #pragma unroll
@@ -155,11 +172,12 @@ APC_EXPORT int apc_conv_heads(const void* proj, int in_dtype, int ld, int q_off,
                               int n_segs, int H, int G, int dk, int dv, const float* bias, const float* conv_w,
                               int taps, float* state, int width, const int* row_seg, const int* seg_row0,
                               const int* seg_rows, const int* slots, const int* positions, int unit_norm, float eps,
-                              int norm_dim, const float* q_norm_w, const float* k_norm_w,
+                              int norm_dim, const float* q_norm_w, const float* k_norm_w, int norm_rows,
+                              float qt_coef, int qt_every,
                               void* q_out, int q_dtype, int ldq, const int* block_table, int max_blocks, void* cache,
                               int cache_dtype, int page_tokens, hipStream_t stream) {
   if (n_rows <= 0) return 0;
-  if (norm_dim < 0 || (norm_dim > 0 && dk % norm_dim)) return APC_ERR_BAD_ARG;
+  if (norm_dim < 0 || (norm_dim > 0 && dk % norm_dim) || qt_every < 0 || (norm_rows && !unit_norm)) return APC_ERR_BAD_ARG;
   if (H <= 0 || G < 0 || dk <= 0 || (G > 0 && dv <= 0) || taps < 1 || width <= 0 || n_segs <= 0) return APC_ERR_BAD_ARG;
   if (taps > 1 && (!conv_w || !state)) return APC_ERR_BAD_ARG;
   if (G > 0 && (!cache || !block_table || page_tokens <= 0 || max_blocks <= 0)) return APC_ERR_BAD_ARG;
@@ -167,7 +185,8 @@ APC_EXPORT int apc_conv_heads(const void* proj, int in_dtype, int ld, int q_off,
     return APC_ERR_UNSUPPORTED;
   hipLaunchKernelGGL(conv_heads_kernel, dim3(n_rows, H + 2 * G), dim3(64), 0, stream, proj, in_dtype, ld, q_off,
                      k_off, v_off, H, G, dk, dv, bias, conv_w, taps, state, width, row_seg, seg_row0, slots, positions,
-                     unit_norm, eps, norm_dim, q_norm_w, k_norm_w, q_out, q_dtype, ldq, block_table, max_blocks, cache, cache_dtype, page_tokens);
+                     unit_norm, eps, norm_dim, q_norm_w, k_norm_w, norm_rows, qt_coef, qt_every, q_out, q_dtype, ldq,
+                     block_table, max_blocks, cache, cache_dtype, page_tokens);
   APC_LAUNCH_CHECK();
   if (taps > 1) {
     hipLaunchKernelGGL(conv_state_kernel, dim3(ceil_div(width, 256), n_segs), dim3(256), 0, stream, proj, in_dtype,
@@ -201,6 +220,8 @@ APC_EXPORT int apc_conv_state(const void* proj, int in_dtype, int ld, const floa
 // With `key_parts` = M > 1 a key of dk elements is M keys of dk / M side by side, one for each of M maps over the same
 // values: q holds H heads of dk / M elements, head j computes its scores with part j % M of the keys of kv head
 // j / (H / G) (the M heads of a group of M are the maps of one head), and `out` holds H heads of dv.
+// `softcap` c > 0: s_t <- c * tanh(s_t / c).  `bias_r1`, `bias_r2` [H]: s_t <- s_t - r1[h] * ln(1 + r2[h] * (pos - t)), a
+// learned penalty on the distance (behind the cap, if both are asked for).
 // The running maximum starts at the sink's score and the running sum at 1 with a sink (the sink is the first "key"),
 // at -inf and 0 without.
 // ---------------------------------------------------------------------------
@@ -209,7 +230,7 @@ __global__ __launch_bounds__(64) void masked_attention_plain_kernel(
     int dk, int dv, const void* __restrict__ cache, int cache_dtype, int P, const int* __restrict__ block_table,
     int max_blocks, const int* __restrict__ positions, const int* __restrict__ row_seg, int mask, int mask_size,
     int sink, const float* __restrict__ sinks, const void* __restrict__ gate, int gate_dtype, int ldg, float scale,
-    int key_parts) {
+    int key_parts, float softcap, const float* __restrict__ bias_r1, const float* __restrict__ bias_r2) {
   __shared__ float qs[MAX_PER_LANE * WAVE];
   __shared__ float ps[WAVE];
   const int r = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
@@ -240,6 +261,8 @@ __global__ __launch_bounds__(64) void masked_attention_plain_kernel(
       float dot = 0.f;
       for (int i = 0; i < dq; ++i) dot = fmaf(qs[i], load_f(cache, cache_dtype, kb + i), dot);
       s = dot * scale;
+      if (softcap > 0.f) s = softcap * tanhf(s / softcap);
+      if (bias_r1) s -= bias_r1[h] * logf(1.0f + bias_r2[h] * (float)(pos - t));
     }
     const float m_new = fmaxf(m, wave_max(s));   // finite: every group in the range holds a visible key
     const float alpha = expf(m - m_new);
@@ -278,16 +301,18 @@ APC_EXPORT int apc_masked_attention_plain(const void* q, int q_dtype, int ldq, v
                                           int page_tokens, const int* block_table, int max_blocks,
                                           const int* positions, const int* row_seg, int mask, int mask_size, int sink,
                                           const float* sinks, const void* gate, int gate_dtype, int ldg, float scale,
-                                          int key_parts, hipStream_t stream) {
+                                          int key_parts, float softcap, const float* bias_r1, const float* bias_r2,
+                                          hipStream_t stream) {
   if (n_rows <= 0) return 0;
   if (H <= 0 || G <= 0 || H % G || dk <= 0 || dv <= 0 || page_tokens <= 0 || max_blocks <= 0 || mask < 0 || mask > 2 ||
       (mask != 0 && mask_size <= 0) || key_parts < 1 || dk % key_parts || (H / G) % key_parts || (sinks && !sink) ||
-      (gate && ldg < H))
+      (gate && ldg < H) || softcap < 0.f || (!bias_r1) != (!bias_r2))
     return APC_ERR_BAD_ARG;
   if (dk > MAX_PER_LANE * WAVE || dv > MAX_PER_LANE * WAVE || H > 65535) return APC_ERR_UNSUPPORTED;
   hipLaunchKernelGGL(masked_attention_plain_kernel, dim3(n_rows, H), dim3(64), 0, stream, q, q_dtype, ldq, out,
                      out_dtype, ldo, H, G, dk, dv, cache, cache_dtype, page_tokens, block_table, max_blocks, positions,
-                     row_seg, mask, mask_size, sink, sinks, gate, gate_dtype, ldg, scale, key_parts);
+                     row_seg, mask, mask_size, sink, sinks, gate, gate_dtype, ldg, scale, key_parts, softcap, bias_r1,
+                     bias_r2);
   APC_LAUNCH_CHECK();
   return 0;
 }

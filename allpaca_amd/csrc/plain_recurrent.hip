@@ -109,12 +109,16 @@ __global__ __launch_bounds__(NT) void rmsnorm_add_f4_kernel(const float* __restr
 // q, k and v pass silu first.  A block takes one segment x one head x 64 value columns and walks the segment's rows
 // in order; thread (rg, j) keeps rows rg, rg + 4, ... of column j of S in registers.  The sum over a column's rows
 // is added in an order fixed by dk alone.
+// With `rot` > 0 the first rot elements of every q and k head are rotated by the row's position (pairs i, i + rot/2:
+// (x, y) -> (x c - y s, y c + x s), c and s from cos_sin[position][2][rot/2]); k is multiplied by `k_scale` behind the
+// rotation.  Both in 32-bit: what enters the state is never rounded.
 // ---------------------------------------------------------------------------
 template <int RPT>   // rows of S a thread keeps: dk <= 4 * RPT
 __global__ __launch_bounds__(256) void linear_attention_kernel(
     const void* __restrict__ proj, int in_dtype, int ld, int q_off, int k_off, int v_off, int H, int dk, int dv, int act,
     const float* __restrict__ decay, float* __restrict__ state, const int* __restrict__ seg_row0,
-    const int* __restrict__ seg_rows, const int* __restrict__ slots, float* __restrict__ out, int ldo) {
+    const int* __restrict__ seg_rows, const int* __restrict__ slots, float* __restrict__ out, int ldo, int rot,
+    const float* __restrict__ cos_sin, const int* __restrict__ positions, float k_scale) {
   __shared__ float qs[2][4 * RPT], ks[2][4 * RPT];
   __shared__ float red[4][64];
   const int seg = blockIdx.x, h = blockIdx.y, j0 = blockIdx.z * 64;
@@ -137,8 +141,20 @@ __global__ __launch_bounds__(256) void linear_attention_kernel(
       float qv = load_f(proj, in_dtype, row + q_off + (size_t)h * dk + i);
       float kv = load_f(proj, in_dtype, row + k_off + (size_t)h * dk + i);
       if (act) { qv = act_silu(qv, in_dtype); kv = act_silu(kv, in_dtype); }
+      if (i < rot) {
+        const int half = rot / 2;
+        const bool first = i < half;
+        const int f = first ? i : i - half, other = first ? i + half : i - half;
+        const float* cs = cos_sin + (size_t)positions[r0 + t] * rot;
+        const float c = cs[f], sn = cs[half + f];
+        float qo = load_f(proj, in_dtype, row + q_off + (size_t)h * dk + other);
+        float ko = load_f(proj, in_dtype, row + k_off + (size_t)h * dk + other);
+        if (act) { qo = act_silu(qo, in_dtype); ko = act_silu(ko, in_dtype); }
+        qv = first ? qv * c - qo * sn : qv * c + qo * sn;
+        kv = first ? kv * c - ko * sn : kv * c + ko * sn;
+      }
       qs[b][i] = qv;
-      ks[b][i] = kv;
+      ks[b][i] = kv * k_scale;
     }
     float vv = on ? load_f(proj, in_dtype, row + v_off + (size_t)h * dv + col) : 0.f;
     if (act) vv = act_silu(vv, in_dtype);
@@ -164,6 +180,31 @@ __global__ __launch_bounds__(256) void linear_attention_kernel(
       const int i = rg + 4 * ii;
       if (i < dk) S[(size_t)i * dv + col] = s[ii];
     }
+  }
+}
+
+// The same with the mean taken over each group of `group` consecutive elements (a head) for itself: one wave a group.
+// `w` [dim] may be absent; gate_kind 0: times sigmoid(gate), 1: times silu(gate).
+__global__ __launch_bounds__(64) void gated_groupnorm_kernel(const float* __restrict__ o, int ldo_in,
+                                                             const float* __restrict__ w, float eps,
+                                                             const void* __restrict__ gate, int gate_dtype, int ldg,
+                                                             int gate_kind, void* __restrict__ out, int out_dtype,
+                                                             int ldo, int group) {
+  const int r = blockIdx.x, c0 = blockIdx.y * group, lane = threadIdx.x;
+  float ss = 0.f;
+  for (int i = lane; i < group; i += WAVE) {
+    const float v = o[(size_t)r * ldo_in + c0 + i];
+    ss = fmaf(v, v, ss);
+  }
+  const float inv = 1.0f / sqrtf(wave_sum(ss) / (float)group + eps);
+  for (int i = lane; i < group; i += WAVE) {
+    float v = o[(size_t)r * ldo_in + c0 + i] * inv;
+    if (w) v *= w[c0 + i];
+    if (gate) {
+      const float z = load_f(gate, gate_dtype, (size_t)r * ldg + c0 + i);
+      v *= gate_kind == 1 ? z * sigmoid_f(z) : sigmoid_f(z);
+    }
+    store_f(out, out_dtype, (size_t)r * ldo + c0 + i, v);
   }
 }
 
@@ -254,15 +295,18 @@ APC_EXPORT int apc_rmsnorm_add(const void* y, int y_dtype, int ldy, const float*
 APC_EXPORT int apc_linear_attention(const void* proj, int in_dtype, int ld, int q_off, int k_off, int v_off, int H,
                                     int dk, int dv, int act, const float* decay, float* state, int n_segs,
                                     const int* seg_row0, const int* seg_rows, const int* slots, float* out, int ldo,
+                                    int rot, const float* cos_sin, const int* positions, float k_scale,
                                     hipStream_t stream) {
   if (n_segs <= 0) return 0;
   if (H <= 0 || dk <= 0 || dv <= 0 || !decay || !state || !slots || ldo < H * dv) return APC_ERR_BAD_ARG;
+  if (rot < 0 || rot % 2 || rot > dk || (rot && (!cos_sin || !positions))) return APC_ERR_BAD_ARG;
   if (dk > 256 || H > 65535 || n_segs > 0x7fffffff / 1) return APC_ERR_UNSUPPORTED;
   dim3 grid(n_segs, H, ceil_div(dv, 64));
   if (grid.z > 65535) return APC_ERR_UNSUPPORTED;
 #define LA_LAUNCH(RPT_)                                                                                            \
   hipLaunchKernelGGL(linear_attention_kernel<RPT_>, grid, dim3(256), 0, stream, proj, in_dtype, ld, q_off, k_off, \
-                     v_off, H, dk, dv, act, decay, state, seg_row0, seg_rows, slots, out, ldo)
+                     v_off, H, dk, dv, act, decay, state, seg_row0, seg_rows, slots, out, ldo, rot, cos_sin, positions,  \
+                     k_scale)
   if (dk <= 32) LA_LAUNCH(8);
   else if (dk <= 64) LA_LAUNCH(16);
   else if (dk <= 128) LA_LAUNCH(32);
@@ -273,9 +317,19 @@ APC_EXPORT int apc_linear_attention(const void* proj, int in_dtype, int ld, int 
 }
 
 APC_EXPORT int apc_gated_rmsnorm(const float* o, int ldo_in, const float* w, float eps, const void* gate, int gate_dtype,
-                                 int ldg, void* out, int out_dtype, int ldo, int n_rows, int dim, hipStream_t stream) {
+                                 int ldg, void* out, int out_dtype, int ldo, int n_rows, int dim, int group,
+                                 int gate_kind, hipStream_t stream) {
   if (n_rows <= 0) return 0;
   if (dim <= 0 || ldo_in < dim || ldo < dim || (gate && ldg < dim)) return APC_ERR_BAD_ARG;
+  if (group < 0 || (group && dim % group) || gate_kind < 0 || gate_kind > 1) return APC_ERR_BAD_ARG;
+  if (group || !w || gate_kind) {
+    const int g = group ? group : dim;
+    if (dim / g > 65535) return APC_ERR_UNSUPPORTED;
+    hipLaunchKernelGGL(gated_groupnorm_kernel, dim3(n_rows, dim / g), dim3(64), 0, stream, o, ldo_in, w, eps, gate,
+                       gate_dtype, ldg, gate_kind, out, out_dtype, ldo, g);
+    APC_LAUNCH_CHECK();
+    return 0;
+  }
   hipLaunchKernelGGL(gated_rmsnorm_kernel<256>, dim3(n_rows), dim3(256), 0, stream, o, ldo_in, w, eps, gate, gate_dtype,
                      ldg, out, out_dtype, ldo, dim);
   APC_LAUNCH_CHECK();

@@ -3,10 +3,13 @@
 // row's result does not depend on the batch; any element type for rows and matrices.
 //
 //   z [T][N] router logits over N = experts with matrices + identity experts (the last ones)
-//   s = softmax(z);  chosen: the K largest of s + correction (the lower index wins a tie);  weights: s of the chosen
+//   s = softmax(z), or s = sigmoid(z) each for itself (`score` 1);  chosen: the K largest of s + correction (the
+//   lower index wins a tie);  weights: s of the chosen
 //   y[t] = sum_k w[t][k] * (expert e = ids[t][k] has matrices ? Wd_e (a(Wg_e h, Wu_e h)) : h)
 //   a(g, u) = silu(g) * u  (`act` 0), or with g' = min(g, limit), u' = clamp(u, -limit, limit):
 //   g' * sigmoid(alpha g') * (u' + 1)  (`act` 1)
+// With `in_weights` the weight multiplies the expert's input instead of its output: y[t] = sum_k expert(w[t][k] h[t]),
+// formed as a(w g, w u) from the same sums g = Wg h, u = Wu h (the products are linear in h).
 #include "common.h"
 #include <math.h>
 
@@ -17,7 +20,7 @@ constexpr int MAX_TOP = 32;
 
 __global__ __launch_bounds__(64) void route_topk_kernel(const float* __restrict__ z, int ldz,
                                                         const float* __restrict__ correction, int N, int K,
-                                                        int renormalize, int* __restrict__ ids,
+                                                        int renormalize, int score, int* __restrict__ ids,
                                                         float* __restrict__ weights) {
   const int t = blockIdx.x, lane = threadIdx.x;
   float s[MAX_PER_LANE_R], c[MAX_PER_LANE_R];
@@ -33,10 +36,11 @@ __global__ __launch_bounds__(64) void route_topk_kernel(const float* __restrict_
 #pragma unroll
   for (int e = 0; e < MAX_PER_LANE_R; ++e) {
     const int i = lane + e * WAVE;
-    s[e] = i < N ? expf(s[e] - mx) : 0.f;
+    if (score == 1) s[e] = i < N ? 1.0f / (1.0f + expf(-s[e])) : 0.f;
+    else s[e] = i < N ? expf(s[e] - mx) : 0.f;
     sum += s[e];
   }
-  sum = wave_sum(sum);
+  sum = score == 1 ? 1.f : wave_sum(sum);
 #pragma unroll
   for (int e = 0; e < MAX_PER_LANE_R; ++e) {
     const int i = lane + e * WAVE;
@@ -82,7 +86,7 @@ __global__ __launch_bounds__(256) void routed_glu_kernel(const void* __restrict_
                                                          const void* __restrict__ w_gate_up, int w_dtype, int E, int F,
                                                          int D, const int* __restrict__ ids, int K,
                                                          void* __restrict__ act, int act_dtype, int kind, float alpha,
-                                                         float limit) {
+                                                         float limit, const float* __restrict__ in_weights) {
   extern __shared__ float hs[];
   const int pair = blockIdx.x, t = pair / K;
   const int e = ids[pair];
@@ -97,6 +101,7 @@ __global__ __launch_bounds__(256) void routed_glu_kernel(const void* __restrict_
     g = fmaf(hs[i], load_f(w_gate_up, w_dtype, gate_row + i), g);
     u = fmaf(hs[i], load_f(w_gate_up, w_dtype, up_row + i), u);
   }
+  if (in_weights) { g *= in_weights[pair]; u *= in_weights[pair]; }
   float a;
   if (kind == 1) {
     g = fminf(g, limit);
@@ -114,7 +119,7 @@ __global__ __launch_bounds__(256) void routed_down_kernel(const void* __restrict
                                                           int D, const int* __restrict__ ids,
                                                           const float* __restrict__ weights, int K,
                                                           const void* __restrict__ h, int h_dtype, int ldh,
-                                                          float* __restrict__ y, int ldy, int in_lds) {
+                                                          float* __restrict__ y, int ldy, int in_lds, int in_weights) {
   extern __shared__ float as[];        // [K][F], if the row's activations fit (else they are read where they lie)
   const int t = blockIdx.x;
   if (in_lds) {
@@ -142,7 +147,8 @@ __global__ __launch_bounds__(256) void routed_down_kernel(const void* __restrict
     } else {
       v = load_f(h, h_dtype, (size_t)t * ldh + d);
     }
-    total = fmaf(weights[(size_t)t * K + k], v, total);
+    // (with the weights on the inputs an expert's output is added as it is; an identity returns its weighted input)
+    total = (in_weights && e < E) ? total + v : fmaf(weights[(size_t)t * K + k], v, total);
   }
   y[(size_t)t * ldy + d] = total;
 }
@@ -150,39 +156,40 @@ __global__ __launch_bounds__(256) void routed_down_kernel(const void* __restrict
 }  // namespace
 
 APC_EXPORT int apc_route_topk(const float* z, int ldz, const float* correction, int n_rows, int N, int K,
-                              int renormalize, int* ids, float* weights, hipStream_t stream) {
+                              int renormalize, int score, int* ids, float* weights, hipStream_t stream) {
   if (n_rows <= 0) return 0;
-  if (N <= 0 || K <= 0 || K > N || ldz < N || !ids || !weights) return APC_ERR_BAD_ARG;
+  if (N <= 0 || K <= 0 || K > N || ldz < N || !ids || !weights || score < 0 || score > 1) return APC_ERR_BAD_ARG;
   if (N > MAX_PER_LANE_R * WAVE || K > MAX_TOP) return APC_ERR_UNSUPPORTED;
-  hipLaunchKernelGGL(route_topk_kernel, dim3(n_rows), dim3(64), 0, stream, z, ldz, correction, N, K, renormalize, ids,
-                     weights);
+  hipLaunchKernelGGL(route_topk_kernel, dim3(n_rows), dim3(64), 0, stream, z, ldz, correction, N, K, renormalize, score,
+                     ids, weights);
   APC_LAUNCH_CHECK();
   return 0;
 }
 
 APC_EXPORT int apc_routed_glu(const void* h, int h_dtype, int ldh, const void* w_gate_up, int w_dtype, int E, int F,
                               int D, const int* ids, int K, void* act, int act_dtype, int n_rows, int kind, float alpha,
-                              float limit, hipStream_t stream) {
+                              float limit, const float* in_weights, hipStream_t stream) {
   if (n_rows <= 0 || E <= 0) return 0;
   if (F <= 0 || D <= 0 || K <= 0 || ldh < D || kind < 0 || kind > 1) return APC_ERR_BAD_ARG;
   if ((size_t)D * sizeof(float) > 64 * 1024 || (long)n_rows * K > 0x7fffffffL || ceil_div(F, 256) > 65535)
     return APC_ERR_UNSUPPORTED;
   hipLaunchKernelGGL(routed_glu_kernel, dim3(n_rows * K, ceil_div(F, 256)), dim3(256), (size_t)D * sizeof(float),
-                     stream, h, h_dtype, ldh, w_gate_up, w_dtype, E, F, D, ids, K, act, act_dtype, kind, alpha, limit);
+                     stream, h, h_dtype, ldh, w_gate_up, w_dtype, E, F, D, ids, K, act, act_dtype, kind, alpha, limit,
+                     in_weights);
   APC_LAUNCH_CHECK();
   return 0;
 }
 
 APC_EXPORT int apc_routed_down(const void* act, int act_dtype, const void* w_down, int w_dtype, int E, int F, int D,
                                const int* ids, const float* weights, int K, const void* h, int h_dtype, int ldh,
-                               float* y, int ldy, int n_rows, hipStream_t stream) {
+                               float* y, int ldy, int n_rows, int in_weights, hipStream_t stream) {
   if (n_rows <= 0) return 0;
   if (E < 0 || F <= 0 || D <= 0 || K <= 0 || ldh < D || ldy < D) return APC_ERR_BAD_ARG;
   if (ceil_div(D, 256) > 65535) return APC_ERR_UNSUPPORTED;
   const size_t lds = (size_t)K * F * sizeof(float);
   const int in_lds = lds <= 48 * 1024 ? 1 : 0;       // (the same sums in the same order either way)
   hipLaunchKernelGGL(routed_down_kernel, dim3(n_rows, ceil_div(D, 256)), dim3(256), in_lds ? lds : 0, stream, act,
-                     act_dtype, w_down, w_dtype, E, F, D, ids, weights, K, h, h_dtype, ldh, y, ldy, in_lds);
+                     act_dtype, w_down, w_dtype, E, F, D, ids, weights, K, h, h_dtype, ldh, y, ldy, in_lds, in_weights);
   APC_LAUNCH_CHECK();
   return 0;
 }

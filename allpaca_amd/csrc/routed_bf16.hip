@@ -16,6 +16,9 @@
 //   down      the same over the activations at their sorted places; float32 out.
 //   combine   y[row] = sum_k weight[row][k] * (down's row at the pair's place, or the input row for an identity
 //             expert), k in order.
+// With the weights on the experts' inputs (`in_weights`: y[row] = sum_k expert(weight * h)) the streaming kernel
+// multiplies the float32 sums of gate and up with the pair's weight ahead of the activation (the products are linear
+// in h), the copy for the tiled kernel writes weight * h, and the last kernel adds the experts' outputs as they are.
 // Experts' matrices: gate_up [E][2][bands(F)][chunks(D)][64][8] and down [E][bands(D)][chunks(F)][64][8] in the tiled
 // layout of the other products.  The grid is made for the most tiles the step can have; a block beyond the tiles that
 // exist leaves at once.
@@ -88,7 +91,7 @@ __global__ __launch_bounds__(256) void routed_glu_bf16_kernel(const bf16_t* __re
                                                               const int* __restrict__ tiles,
                                                               const int* __restrict__ n_tiles,
                                                               bf16_t* __restrict__ act, int kind, float alpha,
-                                                              float limit) {
+                                                              float limit, const float* __restrict__ in_weights) {
   const int ti = blockIdx.x;
   if (ti >= *n_tiles) return;
   const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE, li = lane % 16, lc = lane / 16;
@@ -148,8 +151,9 @@ __global__ __launch_bounds__(256) void routed_glu_bf16_kernel(const bf16_t* __re
     if (!on[rt] || f0 >= F) continue;
     bf16_t* dst = act + (size_t)(p0 + rt * 16 + li) * F + f0;
     float v[4];
+    const float w = in_weights ? in_weights[order[p0 + rt * 16 + li]] : 1.f;
 #pragma unroll
-    for (int r = 0; r < 4; ++r) v[r] = unit_act(g[rt][r], u[rt][r], kind, alpha, limit);
+    for (int r = 0; r < 4; ++r) v[r] = unit_act(g[rt][r] * w, u[rt][r] * w, kind, alpha, limit);
     if (f0 + 4 <= F && F % 4 == 0) {
       uint2 pk;
       pk.x = pack_bf16x2(v[0], v[1]);
@@ -225,28 +229,37 @@ __global__ __launch_bounds__(256) void routed_gather_kernel(const bf16_t* __rest
                                                             const int* __restrict__ order, int K,
                                                             const int* __restrict__ tiles,
                                                             const int* __restrict__ n_tiles, int tile_rows,
-                                                            bf16_t* __restrict__ hs) {
+                                                            bf16_t* __restrict__ hs,
+                                                            const float* __restrict__ in_weights) {
   const int ti = blockIdx.x;
   if (ti >= *n_tiles) return;
   const int p0 = tiles[3 * ti + 1], rows = tiles[3 * ti + 2];
   const int pieces = D / 8;
   for (int idx = blockIdx.y * 256 + threadIdx.x; idx < rows * pieces; idx += gridDim.y * 256) {
     const int r = idx / pieces, c = (idx % pieces) * 8;
-    *reinterpret_cast<Frag*>(hs + (size_t)(p0 + r) * D + c) = load_frag(h + (size_t)(order[p0 + r] / K) * ldh + c);
+    const int pair = order[p0 + r];
+    Frag f = load_frag(h + (size_t)(pair / K) * ldh + c);
+    if (in_weights) {
+      const float w = in_weights[pair];
+#pragma unroll
+      for (int k = 0; k < 4; ++k)
+        f.w[k] = pack_bf16x2(__uint_as_float(f.w[k] << 16) * w, __uint_as_float(f.w[k] & 0xffff0000u) * w);
+    }
+    *reinterpret_cast<Frag*>(hs + (size_t)(p0 + r) * D + c) = f;
   }
 }
 
 __global__ __launch_bounds__(256) void routed_combine_kernel(const float* __restrict__ ys, const int* __restrict__ place,
                                                              const float* __restrict__ weights, int K,
                                                              const bf16_t* __restrict__ h, int ldh,
-                                                             float* __restrict__ y, int ldy, int D) {
+                                                             float* __restrict__ y, int ldy, int D, int in_weights) {
   const int t = blockIdx.x;
   for (int d = threadIdx.x; d < D; d += 256) {
     float total = 0.f;
     for (int k = 0; k < K; ++k) {
       const int at = place[(size_t)t * K + k];
       const float v = at >= 0 ? ys[(size_t)at * D + d] : bf16_to_float(h[(size_t)t * ldh + d]);
-      total = fmaf(weights[(size_t)t * K + k], v, total);
+      total = (in_weights && at >= 0) ? total + v : fmaf(weights[(size_t)t * K + k], v, total);
     }
     y[(size_t)t * ldy + d] = total;
   }
@@ -274,7 +287,7 @@ extern "C" int apc_gemm_grouped_bf16(const void* A, int lda, const void* W, cons
 APC_EXPORT int apc_routed_experts_bf16(const void* h, int ldh, const void* w_gate_up, const void* w_down, int E, int F,
                                        int D, const int* ids, const float* weights, int K, int n_rows, int tile_rows,
                                        int* work, void* act, float* ys, void* hs, float* y, int ldy, int kind,
-                                       float alpha, float limit, hipStream_t stream) {
+                                       float alpha, float limit, int in_weights, hipStream_t stream) {
   if (n_rows <= 0) return 0;
   if (!apc_routed_bf16_takes(E, F, D)) return APC_ERR_UNSUPPORTED;
   if (kind < 0 || kind > 1) return APC_ERR_BAD_ARG;
@@ -296,7 +309,8 @@ APC_EXPORT int apc_routed_experts_bf16(const void* h, int ldh, const void* w_gat
   if (g1.y > 65535 || g2.y > 65535) return APC_ERR_UNSUPPORTED;
   if (tile_rows == 16) {
     hipLaunchKernelGGL(routed_glu_bf16_kernel<1>, g1, dim3(256), 0, stream, (const bf16_t*)h, ldh,
-                       (const bf16_t*)w_gate_up, F, D, order, K, tiles, n_tiles, (bf16_t*)act, kind, alpha, limit);
+                       (const bf16_t*)w_gate_up, F, D, order, K, tiles, n_tiles, (bf16_t*)act, kind, alpha, limit,
+                       in_weights ? weights : nullptr);
     APC_LAUNCH_CHECK();
     hipLaunchKernelGGL(routed_down_bf16_kernel<1>, g2, dim3(256), 0, stream, (const bf16_t*)act, F, D,
                        (const bf16_t*)w_down, tiles, n_tiles, ys);
@@ -304,7 +318,7 @@ APC_EXPORT int apc_routed_experts_bf16(const void* h, int ldh, const void* w_gat
   } else {
     if (max_tiles > 65535) return APC_ERR_UNSUPPORTED;
     hipLaunchKernelGGL(routed_gather_kernel, dim3(max_tiles, 16), dim3(256), 0, stream, (const bf16_t*)h, ldh, D, order, K,
-                       tiles, n_tiles, tile_rows, (bf16_t*)hs);
+                       tiles, n_tiles, tile_rows, (bf16_t*)hs, in_weights ? weights : nullptr);
     APC_LAUNCH_CHECK();
     const size_t gate_elems = (size_t)ceil_div(F, 16) * ceil_div(D, 32) * TILE_ELEMS;
     const size_t down_elems = (size_t)ceil_div(D, 16) * ceil_div(F, 32) * TILE_ELEMS;
@@ -317,7 +331,7 @@ APC_EXPORT int apc_routed_experts_bf16(const void* h, int ldh, const void* w_gat
     if (e) return e;
   }
   hipLaunchKernelGGL(routed_combine_kernel, dim3(n_rows), dim3(256), 0, stream, ys, place, weights, K,
-                     (const bf16_t*)h, ldh, y, ldy, D);
+                     (const bf16_t*)h, ldh, y, ldy, D, in_weights);
   APC_LAUNCH_CHECK();
   return 0;
 }

@@ -34,23 +34,28 @@ SIGNATURES: Dict[str, Dict[str, list]] = {
         "apc_cast": [P, I, P, I, Z, P],
         "apc_gemm_plain": [P, I, I, P, I, I, P, I, I, I, I, I, I, P],
         "apc_paged_attention_plain": [P, I, I, I, P, I, I, I, I, I, I, P, I, I, P, I, P, P, I, F, P],
-        "apc_conv_heads": [P, I, I, I, I, I, I, I, I, I, I, I, P, P, I, P, I, P, P, P, P, P, I, F, I, P, P, P, I, I, P, I, P, I, I, P],
+        "apc_conv_heads": [P, I, I, I, I, I, I, I, I, I, I, I, P, P, I, P, I, P, P, P, P, P, I, F, I, P, P, I, F, I, P, I, I, P, I, P, I, I, P],
         "apc_conv_state": [P, I, I, P, I, P, I, I, P, P, P, P],
-        "apc_masked_attention_plain": [P, I, I, P, I, I, I, I, I, I, I, P, I, I, P, I, P, P, I, I, I, P, P, I, I, F, I, P],
+        "apc_masked_attention_plain": [P, I, I, P, I, I, I, I, I, I, I, P, I, I, P, I, P, P, I, I, I, P, P, I, I, F, I, F, P, P, P],
         "apc_rotary_pages": [P, I, I, I, I, I, I, P, I, I, P, I, I, I, I, P, I, I, I, I, I, I, P, I, I, I, I, I, I, P, P, P,
-                             P, I, P, I, I, I, P],
+                             P, I, P, I, I, I, P, P, F, P],
         "apc_streams_step": [P, I, I, I, P, I, I, P, P, P, P, F, P, I, I, P, P],
         "apc_embed_streams": [P, I, P, P, F, P, I, I, I, P],
         "apc_clamped_glu": [P, I, I, P, I, I, I, I, F, F, P],
         "apc_scale": [P, F, Z, P],
         "apc_embed_positions": [P, I, P, P, I, P, F, P, I, I, I, P],
         "apc_rmsnorm_add": [P, I, I, P, F, F, P, I, P, I, I, I, I, P],
-        "apc_linear_attention": [P, I, I, I, I, I, I, I, I, I, P, P, I, P, P, P, P, I, P],
-        "apc_gated_rmsnorm": [P, I, P, F, P, I, I, P, I, I, I, I, P],
+        "apc_linear_attention": [P, I, I, I, I, I, I, I, I, I, P, P, I, P, P, P, P, I, I, P, P, F, P],
+        "apc_gated_rmsnorm": [P, I, P, F, P, I, I, P, I, I, I, I, I, I, P],
         "apc_diff_combine": [P, I, F, F, F, P, I, I, P, I, I, I, I, I, P],
-        "apc_route_topk": [P, I, P, I, I, I, I, P, P, P],
-        "apc_routed_glu": [P, I, I, P, I, I, I, I, P, I, P, I, I, I, F, F, P],
-        "apc_routed_down": [P, I, P, I, I, I, I, P, P, I, P, I, I, P, I, I, P],
+        "apc_route_topk": [P, I, P, I, I, I, I, I, P, P, P],
+        "apc_routed_glu": [P, I, I, P, I, I, I, I, P, I, P, I, I, I, F, F, P, P],
+        "apc_conv_channels": [P, I, I, I, I, P, P, I, P, P, P, P, I, P, I, I, P],
+        "apc_selective_scan": [P, I, I, P, I, P, P, P, I, P, P, I, I, P, I, I, I, P, P, P, P, I, I, P],
+        "apc_act_rows": [P, I, I, P, I, I, I, I, I, P],
+        "apc_bias_rows": [P, I, P, I, I, P],
+        "apc_weighted_pair": [P, I, P, I, F, P, I, F, I, I, P],
+        "apc_routed_down": [P, I, P, I, I, I, I, P, P, I, P, I, I, P, I, I, I, P],
         "apc_argmax_rows": [P, I, I, I, P, P, P],
         "apc_argmax_rows_no_alloc": [P, I, I, I, P, P],
         "apc_sample_rows": [P, I, I, I, P, P, P, P, P, P, Z, I, P],
@@ -80,7 +85,7 @@ SIGNATURES: Dict[str, Dict[str, list]] = {
         "apc_conv_heads_bf16": [P, I, I, I, I, I, I, P, P, I, P, I, I, P, P, P, P, I, F, I, P, P, P, I, P, I, P, I, P],
         "apc_routed_bf16_takes": [I, I, I],
         "apc_routed_max_tiles": [I, I, I],
-        "apc_routed_experts_bf16": [P, I, P, P, I, I, I, P, P, I, I, I, P, P, P, P, P, I, I, F, F, P],
+        "apc_routed_experts_bf16": [P, I, P, P, I, I, I, P, P, I, I, I, P, P, P, P, P, I, I, F, F, I, P],
         "apc_linear_attention_bf16_takes": [I, I, I, I, I, I, I],
         "apc_linear_attention_bf16": [P, I, I, I, I, I, I, I, I, P, P, I, P, P, P, I, P, P, P, P, I, P],
         "apc_attention_masked_takes": [I, I, I, I, I, I],

@@ -380,16 +380,23 @@ def conv_heads(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, n_heads: 
                state: Optional[torch.Tensor], step, slots: Optional[torch.Tensor], unit_norm: bool, eps: float,
                q_out: torch.Tensor, block_table: Optional[torch.Tensor] = None, cache: Optional[torch.Tensor] = None,
                page_tokens: int = 0, norm_dim: int = 0, q_norm_w: Optional[torch.Tensor] = None,
-               k_norm_w: Optional[torch.Tensor] = None) -> None:
+               k_norm_w: Optional[torch.Tensor] = None, norm_rows: bool = False, q_temp_coef: float = 0.0,
+               q_temp_every: int = 0) -> None:
     """Bias, short causal convolution over time (taps = conv_w.shape[1]; the inputs of the positions ahead of a
     segment come from `state` [slots + 1, taps - 1, width], which is moved on), unit RMS norm of q and k heads,
     q to `q_out` [rows, heads * key_dim], k and v into the pages.  `n_kv_heads` = 0: the row holds q only.
     `norm_dim` (divides key_dim; 0: key_dim): the norm is taken over every piece of that many elements of a head;
-    `q_norm_w`, `k_norm_w` float32 [norm_dim]: weights the normed pieces are multiplied with."""
+    `q_norm_w`, `k_norm_w` float32 [norm_dim]: weights the normed pieces are multiplied with.
+    `norm_rows`: the norm is taken over all heads of q (of k) at once, and the weights are float32
+    [heads * key_dim] ([kv heads * key_dim]).  `q_temp_every` > 0: q of a row at position p is multiplied by
+    1 + q_temp_coef * ln(floor((p + 1) / q_temp_every) + 1)."""
     _gpu(proj, bias, conv_w, state, slots, q_out, block_table, cache, q_norm_w, k_norm_w)
     nd = int(norm_dim) or key_dim
     _need(nd > 0 and key_dim % nd == 0, "conv_heads: norm_dim must divide key_dim")
     _need((q_norm_w is None and k_norm_w is None) or unit_norm, "conv_heads: norm weights need the norm")
+    _need(not norm_rows or (unit_norm and nd == key_dim), "conv_heads: a norm over the whole projection has no pieces")
+    _need(int(q_temp_every) >= 0, "conv_heads: q_temp_every must not be negative")
+    nq, nk = (n_heads * key_dim, int(n_kv_heads) * key_dim) if norm_rows else (nd, nd)
     ld, ldq = _rows(proj, "projected rows"), _rows(q_out, "q out")
     T, width = proj.shape
     G = int(n_kv_heads)
@@ -415,6 +422,7 @@ def conv_heads(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, n_heads: 
     S = step.n_segs
     L = _lib.load("plain")
     if (_tuned_ok(proj, q_out) and (cache is None or cache.dtype == torch.bfloat16) and q_off == 0
+            and not norm_rows and not q_temp_every
             and (G == 0 or (k_off == n_heads * key_dim and v_off == (n_heads + G) * key_dim))):
         LT = _lib.load("tuned")
         if (LT.apc_conv_heads_bf16_takes(ld, width, n_heads, G, key_dim, value_dim, taps, ldq) and nd % 8 == 0
@@ -446,7 +454,8 @@ def conv_heads(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, n_heads: 
         state.data_ptr() if taps > 1 else 0, width, _i32(step.row_seg, T, "row_seg"), _i32(step.seg_row0, S, "seg_row0"),
         _i32(step.seg_rows, S, "seg_rows"), _i32(slots, S, "slots") if taps > 1 else 0,
         _i32(step.positions, T, "positions"), 1 if unit_norm else 0, float(eps), nd,
-        _f32(q_norm_w, nd, "q norm weight"), _f32(k_norm_w, nd, "k norm weight"), q_out.data_ptr(), _code(q_out), ldq,
+        _f32(q_norm_w, nq, "q norm weight"), _f32(k_norm_w, nk, "k norm weight"), 1 if norm_rows else 0,
+        float(q_temp_coef), int(q_temp_every), q_out.data_ptr(), _code(q_out), ldq,
         block_table.data_ptr() if G else 0, max_blocks, cache.data_ptr() if G else 0, _code(cache) if G else 0,
         page_tokens, _stream()), "conv_heads")
 
@@ -455,8 +464,12 @@ def masked_attention_plain(q: torch.Tensor, out: torch.Tensor, n_heads: int, n_k
                            value_dim: int, cache: torch.Tensor, page_tokens: int, block_table: torch.Tensor,
                            positions: torch.Tensor, row_seg: torch.Tensor, mask: str, mask_size: int, sink: bool,
                            scale: float, key_parts: int = 1, sinks: Optional[torch.Tensor] = None,
-                           gate: Optional[torch.Tensor] = None) -> None:
+                           gate: Optional[torch.Tensor] = None, softcap: float = 0.0,
+                           distance_bias: Optional[tuple] = None) -> None:
     _gpu(q, out, cache, block_table, positions, row_seg, sinks, gate)
+    r1, r2 = distance_bias if distance_bias is not None else (None, None)
+    _gpu(r1, r2)
+    _need(float(softcap) >= 0.0, "attention: the soft cap must not be negative")
     ldq, ldo = _rows(q, "attention q"), _rows(out, "attention out")
     T = q.shape[0]
     _check_key_parts(n_heads, n_kv_heads, key_dim, key_parts)
@@ -473,7 +486,8 @@ def masked_attention_plain(q: torch.Tensor, out: torch.Tensor, n_heads: int, n_k
         _i32(positions, T, "positions"), _i32(row_seg, T, "row_seg"), MASKS[mask], int(mask_size), 1 if sink else 0,
         _f32(sinks, n_heads, "sinks"), gate.data_ptr() if gate is not None else 0,
         _code(gate) if gate is not None else 0, _rows(gate, "head gate") if gate is not None else 0,
-        float(scale), int(key_parts), _stream()), "masked_attention_plain")
+        float(scale), int(key_parts), float(softcap), _f32(r1, n_heads, "distance bias r1"),
+        _f32(r2, n_heads, "distance bias r2"), _stream()), "masked_attention_plain")
 
 
 def _check_sinks_gate(sink: bool, sinks, gate, T: int, n_heads: int) -> None:
@@ -491,33 +505,40 @@ def _check_key_parts(n_heads: int, n_kv_heads: int, key_dim: int, key_parts: int
 def masked_attention(q: torch.Tensor, out: torch.Tensor, n_heads: int, n_kv_heads: int, key_dim: int, value_dim: int,
                      cache: torch.Tensor, page_tokens: int, block_table: torch.Tensor, step, mask: str = "causal",
                      mask_size: int = 0, sink: bool = False, scale: float = 1.0, key_parts: int = 1,
-                     sinks: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None) -> None:
+                     sinks: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None, softcap: float = 0.0,
+                     distance_bias: Optional[tuple] = None) -> None:
     """`key_parts` = M > 1: a cached key of `key_dim` elements is M keys of key_dim / M side by side, one for each of M
     softmax maps over the same values; q holds `n_heads` heads of key_dim / M, head j uses part j % M (M consecutive
     heads are the maps of one head), and `out` holds n_heads heads of value_dim (float32 or the run's type).
     `sinks` float32 [heads]: the sink's score per head (0 without).  `gate` [rows, >= heads] logits: head h of a row
-    leaves multiplied by sigmoid(gate[row][h])."""
+    leaves multiplied by sigmoid(gate[row][h]).  `softcap` c > 0: a score s becomes c * tanh(s / c).  `distance_bias`
+    (r1, r2), float32 [heads] each: the score of a key d positions back is lowered by r1[h] * ln(1 + r2[h] * d)."""
     if _tuned_ok(q, cache) and out.dtype in (torch.bfloat16, torch.float32):
         from . import tuned
         if tuned.masked_attention_bf16(q, out, n_heads, n_kv_heads, key_dim, value_dim, cache, page_tokens,
-                                       block_table, step, mask, mask_size, sink, scale, key_parts, sinks, gate):
+                                       block_table, step, mask, mask_size, sink, scale, key_parts, sinks, gate,
+                                       softcap, distance_bias):
             return
     masked_attention_plain(q, out, n_heads, n_kv_heads, key_dim, value_dim, cache, page_tokens, block_table,
-                           step.positions, step.row_seg, mask, mask_size, sink, scale, key_parts, sinks, gate)
+                           step.positions, step.row_seg, mask, mask_size, sink, scale, key_parts, sinks, gate,
+                           softcap, distance_bias)
 
 
 def rotary_pages(q: torch.Tensor, q_off: int, n_heads: int, q_dim: int, q_rot0: int, q_out: torch.Tensor,
                  ka: torch.Tensor, ka_off: int, a_dim: int, kb: Optional[torch.Tensor], kb_off: int, b_dim: int,
                  kb_shared: bool, k_rot0: int, v: torch.Tensor, v_off: int, value_dim: int, n_kv_heads: int, rot: int,
                  cos_sin: Optional[torch.Tensor], step, block_table: torch.Tensor, cache: torch.Tensor,
-                 page_tokens: int) -> None:
+                 page_tokens: int, q_norm_w: Optional[torch.Tensor] = None, k_norm_w: Optional[torch.Tensor] = None,
+                 norm_eps: float = 0.0) -> None:
     """Heads put together, rotated and cached.  Query head h: q[:, q_off + h * q_dim ...], its elements
     [q_rot0, q_rot0 + rot) rotated by the row's position, to q_out [rows, heads * q_dim] (q_out may be q).  Key of kv
     head g: a_dim elements of ka (column ka_off + g * a_dim) followed by b_dim elements of kb (column kb_off, the same
     for every head if `kb_shared`, else + g * b_dim); elements [k_rot0, k_rot0 + rot) of the whole rotated; into the
     pages.  Value of kv head g: v[:, v_off + g * value_dim ...] as it is (it may be the key's own columns).  Pairs are
-    (i, i + rot/2) of the rotated range; cos_sin float32 [positions, 2, rot/2]."""
-    _gpu(q, q_out, ka, kb, v, cos_sin, block_table, cache)
+    (i, i + rot/2) of the rotated range; cos_sin float32 [positions, 2, rot/2].  `q_norm_w` float32 [q_dim],
+    `k_norm_w` float32 [a_dim + b_dim]: the head is first divided by its root mean square (`norm_eps` inside the root)
+    and multiplied with these weights, which all heads share; values are taken as they are."""
+    _gpu(q, q_out, ka, kb, v, cos_sin, block_table, cache, q_norm_w, k_norm_w)
     T = q.shape[0]
     H, G, dq, da, db, dv = int(n_heads), int(n_kv_heads), int(q_dim), int(a_dim), int(b_dim), int(value_dim)
     ldq, ldqo, ldka, ldv = _rows(q, "q"), _rows(q_out, "q out"), _rows(ka, "keys"), _rows(v, "values")
@@ -536,7 +557,7 @@ def rotary_pages(q: torch.Tensor, q_off: int, n_heads: int, q_dim: int, q_rot0: 
     _split_pages(cache, G, da + db, dv, page_tokens)
     _need(block_table.dim() == 2 and block_table.dtype == torch.int32 and block_table.is_contiguous(),
           "block table must be contiguous int32 [segments, blocks]")
-    if _tuned_ok(q, q_out, ka, v, cache):
+    if _tuned_ok(q, q_out, ka, v, cache) and q_norm_w is None and k_norm_w is None:
         from . import tuned
         if tuned.rotary_pages_bf16(q, ldq, q_off, H, dq, q_rot0, q_out, ldqo, ka, ldka, ka_off, da, kb, ldkb, kb_off,
                                    db, kb_shared, k_rot0, v, ldv, v_off, dv, G, rot, cos_sin, step, block_table, cache,
@@ -549,7 +570,8 @@ def rotary_pages(q: torch.Tensor, q_off: int, n_heads: int, q_dim: int, q_rot0: 
         _code(kb) if kb is not None else 0, ldkb, kb_off, db, 1 if kb_shared else 0, k_rot0,
         v.data_ptr(), _code(v), ldv, v_off, dv, G, rot, cos_sin.data_ptr() if rot else 0,
         _i32(step.positions, T, "positions"), _i32(step.row_seg, T, "row_seg"), block_table.data_ptr(),
-        block_table.shape[1], cache.data_ptr(), _code(cache), page_tokens, T, _stream()), "rotary_pages")
+        block_table.shape[1], cache.data_ptr(), _code(cache), page_tokens, T, _f32(q_norm_w, dq, "q norm weight"),
+        _f32(k_norm_w, da + db, "k norm weight"), float(norm_eps), _stream()), "rotary_pages")
 
 
 def streams_step(x: torch.Tensor, n_streams: int, y: Optional[torch.Tensor] = None,
@@ -664,12 +686,21 @@ def rmsnorm_add(y: torch.Tensor, weight: torch.Tensor, eps: float, mult: float, 
 # --------------------------------------------------------------------------- linear attention with a decay
 def linear_attention(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, n_heads: int, key_dim: int,
                      value_dim: int, silu: bool, decay: torch.Tensor, state: torch.Tensor, step, slots: torch.Tensor,
-                     out: torch.Tensor, powers: Optional[torch.Tensor] = None) -> None:
+                     out: torch.Tensor, powers: Optional[torch.Tensor] = None, rot: int = 0,
+                     cos_sin: Optional[torch.Tensor] = None, k_scale: float = 1.0) -> None:
     """Per head S <- decay * S + k_t v_t^T, o_t = S^T q_t over the rows of every segment in order, S float32
     [slots + 1, heads, key_dim, value_dim] per request; q, k, v (through silu if asked) from the projected rows;
     `out` float32 [rows, heads * value_dim].  `powers` (optional): `tuned.decay_powers` of the same decay, kept by the
-    caller for the kernel that walks prompt portions in chunks."""
-    _gpu(proj, decay, state, slots, out, powers)
+    caller for the kernel that walks prompt portions in chunks.  `rot` > 0: the first rot elements of every q and k
+    head are rotated by the row's position (pairs i, i + rot/2; cos_sin float32 [positions, 2, rot/2]); `k_scale`
+    multiplies k behind the rotation."""
+    _gpu(proj, decay, state, slots, out, powers, cos_sin)
+    rot = int(rot)
+    _need(rot % 2 == 0 and 0 <= rot <= int(key_dim), "linear attention: the rotated width must be even and at most key_dim")
+    if rot:
+        _need(cos_sin is not None and cos_sin.dtype == torch.float32 and cos_sin.is_contiguous()
+              and cos_sin.dim() == 3 and cos_sin.shape[1] == 2 and cos_sin.shape[2] == rot // 2,
+              "cos/sin table must be float32 [positions, 2, rot/2]")
     ld, ldo = _rows(proj, "projected rows"), _rows(out, "linear attention out")
     T, width = proj.shape
     H, dk, dv = int(n_heads), int(key_dim), int(value_dim)
@@ -679,7 +710,7 @@ def linear_attention(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, n_h
     _need(state.dtype == torch.float32 and state.is_contiguous() and tuple(state.shape[1:]) == (H, dk, dv),
           f"linear attention: state must be float32 [slots, {H}, {dk}, {dv}]")
     S = step.n_segs
-    if _tuned_ok(proj):
+    if _tuned_ok(proj) and not rot and float(k_scale) == 1.0:
         from . import tuned
         if tuned.linear_attention_bf16(proj, q_off, k_off, v_off, H, dk, dv, silu, decay, state, step, slots, out,
                                        powers):
@@ -688,21 +719,30 @@ def linear_attention(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, n_h
     _lib.check(L.apc_linear_attention(proj.data_ptr(), _code(proj), ld, q_off, k_off, v_off, H, dk, dv,
                                       1 if silu else 0, _f32(decay, H, "decay"), state.data_ptr(), S,
                                       _i32(step.seg_row0, S, "seg_row0"), _i32(step.seg_rows, S, "seg_rows"),
-                                      _i32(slots, S, "slots"), out.data_ptr(), ldo, _stream()), "linear_attention")
+                                      _i32(slots, S, "slots"), out.data_ptr(), ldo, rot,
+                                      cos_sin.data_ptr() if rot else 0, _i32(step.positions, T, "positions") if rot else 0,
+                                      float(k_scale), _stream()), "linear_attention")
 
 
-def gated_rmsnorm(o: torch.Tensor, weight: torch.Tensor, eps: float, gate: Optional[torch.Tensor],
-                  out: torch.Tensor) -> None:
-    """out = rms_norm(o) * weight * sigmoid(gate), the norm over the whole row; o float32, gate (logits) and out any."""
+GATES = {"sigmoid": 0, "silu": 1}
+
+
+def gated_rmsnorm(o: torch.Tensor, weight: Optional[torch.Tensor], eps: float, gate: Optional[torch.Tensor],
+                  out: torch.Tensor, group: int = 0, gate_act: str = "sigmoid") -> None:
+    """out = rms_norm(o) * weight * sigmoid(gate), the norm over the whole row; o float32, gate (logits) and out any.
+    `group` > 0: the norm is taken over every `group` consecutive elements (a head) for itself; `weight` may be None;
+    `gate_act` "silu": times gate * sigmoid(gate)."""
     _gpu(o, weight, gate, out)
     T, N = o.shape
+    _need(gate_act in GATES and int(group) >= 0 and (not group or N % int(group) == 0),
+          "gated_rmsnorm: the gate is 'sigmoid' or 'silu', and a group must divide the row")
     _need(o.dtype == torch.float32 and out.shape == (T, N) and (gate is None or gate.shape == (T, N)),
           "gated_rmsnorm: o float32 [rows, n], gate and out of the same shape")
     L = _lib.load("plain")
     _lib.check(L.apc_gated_rmsnorm(o.data_ptr(), _rows(o, "o"), _f32(weight, N, "norm weight"), float(eps),
                                    gate.data_ptr() if gate is not None else 0, _code(gate) if gate is not None else 0,
                                    _rows(gate, "gate") if gate is not None else 0, out.data_ptr(), _code(out),
-                                   _rows(out, "out"), T, N, _stream()), "gated_rmsnorm")
+                                   _rows(out, "out"), T, N, int(group), GATES[gate_act], _stream()), "gated_rmsnorm")
 
 
 def diff_combine(a: torch.Tensor, lam: float, post: float, eps: float, gate: Optional[torch.Tensor],
@@ -723,18 +763,22 @@ def diff_combine(a: torch.Tensor, lam: float, post: float, eps: float, gate: Opt
 
 
 # --------------------------------------------------------------------------- routed experts
+ROUTER_SCORES = {"softmax": 0, "sigmoid": 1}
+
+
 def route_topk(z: torch.Tensor, correction: Optional[torch.Tensor], top: int, ids: torch.Tensor,
-               weights: torch.Tensor, renormalize: bool = False) -> None:
-    """s = softmax(z) over a row; the `top` largest of s + correction are chosen (the lower index wins a tie);
+               weights: torch.Tensor, renormalize: bool = False, score: str = "softmax") -> None:
+    """s = softmax(z) over a row (`score` "sigmoid": s = sigmoid(z), every output for itself); the `top` largest of s + correction are chosen (the lower index wins a tie);
     weights = s of the chosen (divided by their sum with `renormalize`).  z float32 [rows, n]."""
     _gpu(z, correction, ids, weights)
     T, N = z.shape
     _need(z.dtype == torch.float32 and weights.dtype == torch.float32 and weights.is_contiguous()
           and weights.numel() >= T * top, "route_topk: z float32, weights contiguous float32 [rows, top]")
+    _need(score in ROUTER_SCORES, f"route_topk: score {score!r} is not one of {sorted(ROUTER_SCORES)}")
     L = _lib.load("plain")
     _lib.check(L.apc_route_topk(z.data_ptr(), _rows(z, "router logits"), _f32(correction, N, "correction"), T, N,
-                                int(top), 1 if renormalize else 0, _i32(ids, T * top, "ids"), weights.data_ptr(),
-                                _stream()), "route_topk")
+                                int(top), 1 if renormalize else 0, ROUTER_SCORES[score], _i32(ids, T * top, "ids"),
+                                weights.data_ptr(), _stream()), "route_topk")
 
 
 def prepare_experts(gate_up: torch.Tensor, down: torch.Tensor, run_dtype: torch.dtype):
@@ -753,12 +797,13 @@ EXPERT_ACTIVATIONS = {"silu": 0, "clamped": 1}
 
 def routed_experts(h: torch.Tensor, w_gate_up, w_down, n_experts: int, ff: int, ids: torch.Tensor,
                    weights: torch.Tensor, top: int, y: torch.Tensor, activation: str = "silu", alpha: float = 1.0,
-                   limit: float = 0.0) -> None:
+                   limit: float = 0.0, weight_input: bool = False) -> None:
     """y[t] = sum_k weights[t][k] * expert ids[t][k] (h[t]); experts 0 .. n_experts-1 are gated units
     Wd a(Wg h, Wu h) with w_gate_up [n_experts, 2 * ff, width] (gate rows, then up rows) and w_down
     [n_experts, width, ff]; ids from n_experts on are identity experts.  y float32 [rows, width].
     `activation` "silu": a(g, u) = silu(g) * u; "clamped": g' * sigmoid(alpha g') * (u' + 1) with g' = min(g, limit),
-    u' = clamp(u, -limit, limit)."""
+    u' = clamp(u, -limit, limit).  `weight_input`: the weight multiplies the expert's input instead of its output,
+    y[t] = sum_k expert(weights[t][k] * h[t]) (identity experts then return the weighted row as well)."""
     T, D = h.shape
     E, F, K = int(n_experts), int(ff), int(top)
     _gpu(h, ids, weights, y)
@@ -767,7 +812,7 @@ def routed_experts(h: torch.Tensor, w_gate_up, w_down, n_experts: int, ff: int, 
     kind = EXPERT_ACTIVATIONS[activation]
     if not isinstance(w_gate_up, torch.Tensor) and w_gate_up is not None:
         from . import tuned
-        tuned.routed_experts_bf16(h, w_gate_up, w_down, E, F, ids, weights, K, y, kind, alpha, limit)
+        tuned.routed_experts_bf16(h, w_gate_up, w_down, E, F, ids, weights, K, y, kind, alpha, limit, weight_input)
         return
     act = torch.empty((T * K, F), dtype=h.dtype, device=h.device)
     L = _lib.load("plain")
@@ -777,9 +822,114 @@ def routed_experts(h: torch.Tensor, w_gate_up, w_down, n_experts: int, ff: int, 
               and tuple(w_down.shape) == (E, D, F), "routed_experts: matrices [experts, 2 ff, width] and [experts, width, ff]")
         _lib.check(L.apc_routed_glu(h.data_ptr(), _code(h), _rows(h, "h"), w_gate_up.data_ptr(), _code(w_gate_up), E, F,
                                     D, _i32(ids, T * K, "ids"), K, act.data_ptr(), _code(act), T, kind, float(alpha),
-                                    float(limit), _stream()),
+                                    float(limit), _f32(weights, T * K, "weights") if weight_input else 0, _stream()),
                    "routed_glu")
     _lib.check(L.apc_routed_down(act.data_ptr(), _code(act), w_down.data_ptr() if E else 0,
                                  _code(w_down) if E else 0, E, F, D, _i32(ids, T * K, "ids"),
                                  _f32(weights, T * K, "weights"), K, h.data_ptr(), _code(h), _rows(h, "h"),
-                                 y.data_ptr(), _rows(y, "y"), T, _stream()), "routed_down")
+                                 y.data_ptr(), _rows(y, "y"), T, 1 if weight_input else 0, _stream()), "routed_down")
+
+
+# --------------------------------------------------------------------------- selective scan, activations, biases
+ACTIVATIONS = {"none": 0, "silu": 1, "relu2": 2, "gelu_tanh": 3}
+
+
+def conv_channels(x: torch.Tensor, channels: int, conv_w: torch.Tensor, bias: Optional[torch.Tensor],
+                  state: Optional[torch.Tensor], step, slots: Optional[torch.Tensor], activation: str,
+                  out: torch.Tensor) -> None:
+    """A short causal convolution over time on the first `channels` columns of x, the bias behind it, then the
+    activation: out[t][c] = act(sum_j conv_w[c][j] * x[t - (taps - 1) + j][c] + bias[c]) inside a segment; the inputs
+    of the positions ahead of a segment come from `state` float32 [slots + 1, taps - 1, channels], which is moved on to
+    the segment's last inputs."""
+    _gpu(x, conv_w, bias, state, slots, out)
+    ldx, ldo = _rows(x, "conv input"), _rows(out, "conv out")
+    T, C = x.shape[0], int(channels)
+    _need(activation in ACTIVATIONS, f"conv_channels: activation {activation!r} is not one of {sorted(ACTIVATIONS)}")
+    _need(C <= x.shape[1] and out.shape == (T, C), "conv_channels: out must be [rows, channels]")
+    _need(conv_w.dim() == 2 and conv_w.shape[0] == C and conv_w.dtype == torch.float32 and conv_w.is_contiguous(),
+          "conv_channels: weights must be float32 [channels, taps]")
+    taps = int(conv_w.shape[1])
+    S = step.n_segs
+    if taps > 1:
+        _need(state is not None and slots is not None and state.dim() == 3 and state.is_contiguous()
+              and state.dtype == torch.float32 and tuple(state.shape[1:]) == (taps - 1, C),
+              f"conv_channels: state must be float32 [slots, {taps - 1}, {C}]")
+    L = _lib.load("plain")
+    _lib.check(L.apc_conv_channels(x.data_ptr(), _code(x), ldx, T, C, conv_w.data_ptr(), _f32(bias, C, "bias"), taps,
+                                   state.data_ptr() if taps > 1 else 0, _i32(step.row_seg, T, "row_seg"),
+                                   _i32(step.seg_row0, S, "seg_row0"), _i32(slots, S, "slots") if taps > 1 else 0,
+                                   ACTIVATIONS[activation], out.data_ptr(), _code(out), ldo, _stream()),
+               "conv_channels")
+    if taps > 1:
+        _lib.check(L.apc_conv_state(x.data_ptr(), _code(x), ldx, 0, taps, state.data_ptr(), C, S,
+                                    _i32(step.seg_row0, S, "seg_row0"), _i32(step.seg_rows, S, "seg_rows"),
+                                    _i32(slots, S, "slots"), _stream()), "conv_state")
+
+
+def selective_scan(x: torch.Tensor, dt: torch.Tensor, dt_bias: Optional[torch.Tensor], A: torch.Tensor,
+                   bc: torch.Tensor, D: Optional[torch.Tensor], z: torch.Tensor, state: torch.Tensor, step,
+                   slots: torch.Tensor, out: torch.Tensor) -> None:
+    """Per channel c with N states, over the rows of every segment in order:
+      d = softplus(dt[t][c] + dt_bias[c]);  S[c][n] <- exp(d A[c][n]) S[c][n] + d x[t][c] B[t][n]
+      out[t][c] = (sum_n S[c][n] C[t][n] + D[c] x[t][c]) * silu(z[t][c])
+    x, z, out [rows, channels] (any element type), dt float32 [rows, channels], bc float32 [rows, 2 N] (B, then C),
+    A float32 [channels, N], state float32 [slots + 1, channels, N]."""
+    _gpu(x, dt, dt_bias, A, bc, D, z, state, slots, out)
+    T, C = out.shape
+    N = int(A.shape[1])
+    _need(x.shape == (T, C) and z.shape == (T, C) and dt.shape == (T, C) and dt.dtype == torch.float32
+          and bc.shape == (T, 2 * N) and bc.dtype == torch.float32, "selective_scan: x, z, dt [rows, channels], bc float32 [rows, 2 N]")
+    _need(A.dtype == torch.float32 and A.is_contiguous() and tuple(A.shape) == (C, N), "selective_scan: A float32 [channels, N]")
+    _need(state.dtype == torch.float32 and state.is_contiguous() and tuple(state.shape[1:]) == (C, N),
+          f"selective_scan: state must be float32 [slots, {C}, {N}]")
+    S = step.n_segs
+    L = _lib.load("plain")
+    _lib.check(L.apc_selective_scan(x.data_ptr(), _code(x), _rows(x, "x"), dt.data_ptr(), _rows(dt, "dt"),
+                                    _f32(dt_bias, C, "dt bias"), A.data_ptr(), bc.data_ptr(), _rows(bc, "B and C"),
+                                    _f32(D, C, "D"), z.data_ptr(), _code(z), _rows(z, "z"), state.data_ptr(), C, N, S,
+                                    _i32(step.seg_row0, S, "seg_row0"), _i32(step.seg_rows, S, "seg_rows"),
+                                    _i32(slots, S, "slots"), out.data_ptr(), _code(out), _rows(out, "out"), _stream()),
+               "selective_scan")
+
+
+def act_rows(x: torch.Tensor, out: torch.Tensor, activation: str) -> None:
+    """out = act(x) element by element: "silu", "relu2" (the square of max(x, 0)), "gelu_tanh", "none"."""
+    _gpu(x, out)
+    _need(activation in ACTIVATIONS, f"act_rows: activation {activation!r} is not one of {sorted(ACTIVATIONS)}")
+    _need(x.shape == out.shape, "act_rows: shapes differ")
+    ldi, ldo = _rows(x, "act in"), _rows(out, "act out")
+    T, n = x.shape
+    L = _lib.load("plain")
+    _lib.check(L.apc_act_rows(x.data_ptr(), _code(x), ldi, out.data_ptr(), _code(out), ldo, T, n,
+                              ACTIVATIONS[activation], _stream()), "act_rows")
+
+
+def bias_rows(x: torch.Tensor, bias: torch.Tensor) -> None:
+    """x[t] += bias (x float32 [rows, n], bias float32 [n])."""
+    _gpu(x, bias)
+    ldx = _rows(x, "bias x")
+    T, n = x.shape
+    _need(x.dtype == torch.float32, "bias_rows: x float32")
+    L = _lib.load("plain")
+    _lib.check(L.apc_bias_rows(x.data_ptr(), ldx, _f32(bias, n, "bias"), T, n, _stream()), "bias_rows")
+
+
+def weighted_pair(u: torch.Tensor, a: float, v: torch.Tensor, b: float, out: torch.Tensor) -> None:
+    """out = a * u + b * v (float32 rows; out may be u)."""
+    _gpu(u, v, out)
+    T, n = out.shape
+    _need(u.shape == (T, n) and v.shape == (T, n) and all(t.dtype == torch.float32 for t in (u, v, out)),
+          "weighted_pair: three float32 [rows, n]")
+    L = _lib.load("plain")
+    _lib.check(L.apc_weighted_pair(out.data_ptr(), _rows(out, "out"), u.data_ptr(), _rows(u, "u"), float(a),
+                                   v.data_ptr(), _rows(v, "v"), float(b), T, n, _stream()), "weighted_pair")
+
+
+def linear_act(a: torch.Tensor, w, out: torch.Tensor, activation: str) -> None:
+    """out = act(a . w^T): the product's sums are 32-bit, the activation is applied to them before they are stored in
+    `out`'s element type."""
+    _need(activation in ACTIVATIONS, f"linear_act: activation {activation!r} is not one of {sorted(ACTIVATIONS)}")
+    T, n = out.shape
+    sums = torch.empty((T, n), dtype=torch.float32, device=a.device)
+    linear(a, w, sums)
+    act_rows(sums, out, activation)

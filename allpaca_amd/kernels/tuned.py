@@ -462,7 +462,7 @@ MASKED_DECODE_SPLITS = 64     # at most: the adding kernel takes 64 parts
 
 def masked_attention_bf16(q, out, n_heads, n_kv_heads, key_dim, value_dim, cache, page_tokens, block_table, step,
                           mask: str, mask_size: int, sink: bool, scale: float, key_parts: int = 1, sinks=None,
-                          gate=None) -> bool:
+                          gate=None, softcap: float = 0.0, distance_bias=None) -> bool:
     """Attention with a chunked or sliding mask and an optional sink on the MFMA kernels: segments of several rows on
     the tiled kernel, single rows on the kernel that cuts a row's keys into ranges.  False (nothing done) for sizes
     they do not take; the caller then runs the plain kernel."""
@@ -472,6 +472,8 @@ def masked_attention_bf16(q, out, n_heads, n_kv_heads, key_dim, value_dim, cache
     L = _lib.load("tuned")
     f32 = out.dtype == torch.float32
     if gate is not None and gate.dtype != torch.float32:
+        return False
+    if softcap or distance_bias is not None:
         return False
     _ops._check_sinks_gate(sink, sinks, gate, T, n_heads)
     sinks_p = _ops._f32(sinks, n_heads, "sinks")
@@ -593,8 +595,9 @@ def pack_experts(gate_up: torch.Tensor, down: torch.Tensor):
 
 
 def routed_experts_bf16(h, w_gate_up: PackedExperts, w_down: PackedExperts, E: int, F: int, ids, weights, K: int,
-                        y, kind: int = 0, alpha: float = 1.0, limit: float = 0.0) -> None:
-    """The chosen experts of every row on the MFMA kernels (pairs sorted by expert on the GPU, nothing read back)."""
+                        y, kind: int = 0, alpha: float = 1.0, limit: float = 0.0, weight_input: bool = False) -> None:
+    """The chosen experts of every row on the MFMA kernels (pairs sorted by expert on the GPU, nothing read back).
+    `weight_input`: a pair's weight multiplies the expert's input instead of its output."""
     T, D = h.shape
     _ops._gpu(h, w_gate_up.data, w_down.data, ids, weights, y)
     _ops._need(h.dtype == torch.bfloat16 and (w_gate_up.E, w_gate_up.N, w_gate_up.K) == (E, F, D)
@@ -612,7 +615,7 @@ def routed_experts_bf16(h, w_gate_up: PackedExperts, w_down: PackedExperts, E: i
         h.data_ptr(), _ops._rows(h, "h"), w_gate_up.data.data_ptr(), w_down.data.data_ptr(), E, F, D,
         _ops._i32(ids, n_pairs, "ids"), _ops._f32(weights, n_pairs, "weights"), K, T, tile_rows, work.data_ptr(),
         act.data_ptr(), ys.data_ptr(), hs.data_ptr() if hs is not None else 0, y.data_ptr(), _ops._rows(y, "y"),
-        int(kind), float(alpha), float(limit), _ops._stream()),
+        int(kind), float(alpha), float(limit), 1 if weight_input else 0, _ops._stream()),
         "routed_experts_bf16")
 
 

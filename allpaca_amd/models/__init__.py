@@ -49,7 +49,7 @@ def describe_model(config_json: Mapping[str, Any],
     return arch, cfg, spec
 
 
-from . import gulidra, lesarax, llama, risizen  # noqa: E402,F401  (they register themselves)
+from . import gulidra, lesarax, llama, risizen, seredra  # noqa: E402,F401  (they register themselves)
 from .decoder import DecoderModel, load_model  # noqa: E402
 
 __all__ = ["ARCHITECTURES", "Architecture", "architecture_of", "describe_model", "DecoderModel", "load_model"]

@@ -51,7 +51,12 @@ class Block:
             for name, key in (("cache_need", role), ("state_need", role + ".state")):
                 ask = getattr(part, name, None)
                 need = ask() if callable(ask) and not (borrows and name == "cache_need") else None
-                if need is not None:
+                if isinstance(need, dict):
+                    # a part made of several (mixers side by side): its members' needs stand under "<role>.<member>"
+                    for member, n in need.items():
+                        if n is not None:
+                            out[f"{role}.{member}" + (".state" if name == "state_need" else "")] = n
+                elif need is not None:
                     out[key] = need
         return out
 

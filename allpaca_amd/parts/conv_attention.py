@@ -16,10 +16,16 @@ taps - 1 positions are per-request state (float32), kept by the mixer itself als
 `key_parts` = M > 1: a head has M softmax maps over the same values.  `key_dim` then counts all M queries (keys) of a
 head side by side, the unit norm is taken over each of the M pieces, and `attend` returns the M maps' outputs of every
 head side by side in float32 for a subclass to combine (`DifferentialAttention`).  `norm_weights`: the normed pieces of
-q and k are multiplied with the tensors "<q>.norm" and "<k>.norm" [key_dim / M], shared by all heads and maps."""
+q and k are multiplied with the tensors "<q>.norm" and "<k>.norm" [key_dim / M], shared by all heads and maps.
+
+`norm_scope` "projection": the root mean square is taken over all heads of q (of k) at once, before they are split into
+heads, and the weights "<q>.norm", "<k>.norm" have the projection's size.  `q_temp` = (coef, every): q of the row at
+position p is multiplied by 1 + coef * ln(floor((p + 1) / every) + 1).  `distance_bias`: tensors "r1", "r2" [heads];
+the score of a key d positions back is lowered by r1[h] * ln(1 + r2[h] * d).  `out_bias`: the output projection has a
+bias "<o><bias>"."""
 from __future__ import annotations
 
-from typing import Dict, Mapping, Optional
+from typing import Dict, Mapping, Optional, Sequence
 
 import torch
 
@@ -36,7 +42,8 @@ class ConvAttention(Mixer):
                  scale: float, conv_taps: int = 0, unit_norm: bool = True, norm_eps: float = 1e-6, bias: bool = True,
                  mask: str = "causal", mask_size: int = 0, sink: bool = False, shares_kv: bool = False,
                  names: Optional[Mapping[str, str]] = None, key_parts: int = 1, norm_weights: bool = False,
-                 extra_rows: int = 0):
+                 extra_rows: int = 0, norm_scope: str = "head", q_temp: Optional[Sequence[float]] = None,
+                 distance_bias: bool = False, out_bias: bool = False):
         if num_heads % num_kv_heads:
             raise ValueError(f"attention: {num_heads} heads are not a multiple of {num_kv_heads} kv heads")
         if mask not in ops.MASKS or (mask != "causal" and int(mask_size) <= 0):
@@ -51,10 +58,21 @@ class ConvAttention(Mixer):
         self.key_parts, self.norm_weights = int(key_parts), bool(norm_weights)
         if self.key_parts < 1 or self.dk % self.key_parts or (self.norm_weights and not self.unit_norm):
             raise ValueError(f"attention: key_parts {key_parts} must divide key_dim {key_dim}, and norm weights need the norm")
+        if norm_scope not in ("head", "projection") or (norm_scope == "projection" and
+                                                        (not self.unit_norm or self.key_parts != 1)):
+            raise ValueError(f"attention: norm_scope {norm_scope!r} ('head', or 'projection' with the norm and one map a head)")
+        self.norm_rows = norm_scope == "projection"
+        self.q_temp = None
+        if q_temp is not None:
+            coef, every = q_temp
+            if int(every) != every or int(every) <= 0:
+                raise ValueError(f"attention: the query temperature's step {every!r} must be a positive whole number")
+            self.q_temp = (float(coef), int(every))
+        self.distance_bias, self.out_bias = bool(distance_bias), bool(out_bias)
         self.extra_rows = int(extra_rows)      # rows a subclass adds to the input matrix behind q, k and v
         # tensor names: projections q, k, v, o; "<projection><bias>" and "<projection><conv>" beside them
         self.names = {"q": "q", "k": "k", "v": "v", "o": "o", "bias": ".b", "conv": ".conv", "norm": ".norm",
-                      **dict(names or {})}
+                      "r1": "r1", "r2": "r2", **dict(names or {})}
         self.projections = [("q", self.H * self.dk)]
         if not self.shares_kv:
             self.projections += [("k", self.G * self.dk), ("v", self.G * self.dv)]
@@ -71,9 +89,14 @@ class ConvAttention(Mixer):
             if self.taps >= 1:
                 out[n[p] + n["conv"]] = ParamSpec((rows, self.taps), store="float32", init="normal")
         if self.norm_weights:
-            for p, _ in self.projections[:2]:
-                out[n[p] + n["norm"]] = ParamSpec((self.dk // self.key_parts,), store="float32")
+            for p, rows in self.projections[:2]:
+                out[n[p] + n["norm"]] = ParamSpec((rows if self.norm_rows else self.dk // self.key_parts,), store="float32")
+        if self.distance_bias:
+            out[n["r1"]] = ParamSpec((self.H,), store="float32", init=0.5)
+            out[n["r2"]] = ParamSpec((self.H,), store="float32", init=0.5)
         out[n["o"]] = ParamSpec((self.D, self.H * self.dv))
+        if self.out_bias:
+            out[n["o"] + n["bias"]] = ParamSpec((self.D,), store="float32", init="zeros")
         return out
 
     def extra_matrices(self, tensors, rt) -> list:
@@ -104,7 +127,11 @@ class ConvAttention(Mixer):
             mats.append(torch.zeros((self.full_width - self.width - self.extra_rows, self.D), dtype=dt, device=rt.device))
         self.w_in = ops.prepare_matrix(torch.cat(mats, dim=0), rt.dtype)
         self.w_o = ops.prepare_matrix(to_device(tensors[n["o"]], rt), rt.dtype)
-        self.b_in = self.conv_w = None
+        self.b_in = self.conv_w = self.b_o = self.r12 = None
+        if self.out_bias:
+            self.b_o = to_device(tensors[n["o"] + n["bias"]], rt, torch.float32)
+        if self.distance_bias:
+            self.r12 = (to_device(tensors[n["r1"]], rt, torch.float32), to_device(tensors[n["r2"]], rt, torch.float32))
         if self.bias:
             self.b_in = torch.cat([to_device(tensors[n[p] + n["bias"]], rt, torch.float32)
                                    for p, _ in self.projections]).contiguous()
@@ -130,11 +157,14 @@ class ConvAttention(Mixer):
                        self.b_in, self.conv_w, state.state if state is not None else None, step,
                        state.slots if state is not None else None, self.unit_norm, self.eps, q,
                        pages.block_table if own else None, pages.kv if own else None, pages.page_tokens,
-                       norm_dim=self.dk // self.key_parts, q_norm_w=self.q_norm_w, k_norm_w=self.k_norm_w)
+                       norm_dim=self.dk // self.key_parts, q_norm_w=self.q_norm_w, k_norm_w=self.k_norm_w,
+                       norm_rows=self.norm_rows, q_temp_coef=self.q_temp[0] if self.q_temp else 0.0,
+                       q_temp_every=self.q_temp[1] if self.q_temp else 0)
         M = self.key_parts
         attn = torch.empty((T, self.H * M * self.dv), dtype=out_dtype or dt, device=dev)
         ops.masked_attention(q, attn, self.H * M, self.G, self.dk, self.dv, pages.kv, pages.page_tokens,
-                             pages.block_table, step, self.mask, self.mask_size, self.sink, self.scale, key_parts=M)
+                             pages.block_table, step, self.mask, self.mask_size, self.sink, self.scale, key_parts=M,
+                             distance_bias=self.r12)
         return full, attn
 
     def forward(self, h, step, cache) -> torch.Tensor:
@@ -145,6 +175,8 @@ class ConvAttention(Mixer):
         T, dev = attn.shape[0], attn.device
         out = torch.empty((T, self.D), dtype=torch.float32, device=dev)
         ops.linear(attn, self.w_o, out)
+        if self.b_o is not None:
+            ops.bias_rows(out, self.b_o)
         return out
 
 

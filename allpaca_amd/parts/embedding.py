@@ -16,8 +16,9 @@ from .spec import ParamSpec
 class TokenEmbedding(Part):
     graph_safe = True
 
-    def __init__(self, vocab_size: int, hidden_size: int, name: str = "weight"):
+    def __init__(self, vocab_size: int, hidden_size: int, name: str = "weight", scale: float = 1.0):
         self.V, self.D, self.name = int(vocab_size), int(hidden_size), name      # `name`: the table's tensor name
+        self.scale = float(scale)                                                # x = table[token] * scale, in 32-bit
 
     def param_specs(self) -> Dict[str, ParamSpec]:
         return {self.name: ParamSpec((self.V, self.D))}
@@ -28,9 +29,13 @@ class TokenEmbedding(Part):
 
     def forward(self, tokens: torch.Tensor, out: torch.Tensor) -> None:
         ops.embed_rows(self.weight, tokens, out)
+        if self.scale != 1.0:
+            ops.scale_(out, self.scale)
 
     def native_desc(self):
-        return {"kind": "token_table", "weight": self.weight} if type(self) is TokenEmbedding else None
+        if type(self) is not TokenEmbedding or self.scale != 1.0:
+            return None
+        return {"kind": "token_table", "weight": self.weight}
 
 
 @EMBEDDINGS.register("token_table_norm")

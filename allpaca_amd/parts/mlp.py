@@ -99,3 +99,37 @@ class ClampedGLU(FeedForward):
         out = torch.empty((h.shape[0], self.D), dtype=torch.float32, device=h.device)
         ops.linear(act, self.w_down, out)
         return out
+
+
+@FEED_FORWARDS.register("mlp")
+class ActMLP(FeedForward):
+    """Two matrices and an activation between them, no gate and no bias: out = Wd act(Wu h).  `activation`: "relu2"
+    (the square of max(z, 0)), "gelu_tanh" (0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3)))), "silu"."""
+    graph_safe = True
+
+    def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "relu2",
+                 names: Mapping[str, str] | None = None):
+        self.D, self.F = int(hidden_size), int(intermediate_size)
+        if activation not in ops.ACTIVATIONS or activation == "none":
+            raise ValueError(f"mlp: activation {activation!r} is not one of {sorted(set(ops.ACTIVATIONS) - {'none'})}")
+        self.activation = activation
+        self.names = {"up": "up", "down": "down", **dict(names or {})}
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        n = self.names
+        return {n["up"]: ParamSpec((self.F, self.D)), n["down"]: ParamSpec((self.D, self.F))}
+
+    def bind(self, tensors: Mapping[str, torch.Tensor], rt: Runtime) -> None:
+        self.rt = rt
+        n = self.names
+        self.w_up = ops.prepare_matrix(to_device(tensors[n["up"]], rt), rt.dtype)
+        self.w_down = ops.prepare_matrix(to_device(tensors[n["down"]], rt), rt.dtype)
+
+    def forward(self, h, step) -> torch.Tensor:
+        h = as_normed(h).tensor()
+        T, dev = h.shape[0], h.device
+        act = torch.empty((T, self.F), dtype=self.rt.dtype, device=dev)
+        ops.linear_act(h, self.w_up, act, self.activation)
+        out = torch.empty((T, self.D), dtype=torch.float32, device=dev)
+        ops.linear(act, self.w_down, out)
+        return out

@@ -9,6 +9,12 @@ The reference has no frequency scaling on its llama path
 one: by wavelength 2*pi/inv_freq, short waves keep their frequency, long waves
 are slowed by `factor`, and the band between is blended linearly.
 
+The "yarn" rule (keys factor, original, fast, slow; `base` is the encoding's own theta): with
+dim(t) = rot * ln(original / (2 pi t)) / (2 ln base), lo = max(floor(dim(fast)), 0), hi = min(ceil(dim(slow)), rot - 1)
+and ramp_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1), frequency i is f_i / factor * ramp_i + f_i * (1 - ramp_i):
+the fast dimensions keep their frequency, the slow ones are divided by the factor; cosines and sines are both
+multiplied by 0.1 * ln(factor) + 1 (`table_magnitude`).
+
 Angles are formed in 64-bit on the host (position * inv_freq) and the cosines
 and sines rounded once to float32: a table [positions, 2, rot/2]."""
 from __future__ import annotations
@@ -29,8 +35,19 @@ def inverse_frequencies(rot: int, theta: float, scaling: Optional[Mapping] = Non
     if not scaling:
         return inv
     kind = scaling.get("rope_type", "llama3")
+    if kind == "yarn":
+        factor, orig = float(scaling["factor"]), float(scaling["original"])
+        fast, slow = float(scaling["fast"]), float(scaling["slow"])
+
+        def dim_of(turns: float) -> float:
+            return rot * math.log(orig / (2.0 * math.pi * turns)) / (2.0 * math.log(float(theta)))
+
+        lo = max(math.floor(dim_of(fast)), 0)
+        hi = min(math.ceil(dim_of(slow)), rot - 1)
+        ramp = np.clip((i - lo) / max(hi - lo, 0.001), 0.0, 1.0)
+        return inv / factor * ramp + inv * (1.0 - ramp)
     if kind != "llama3":
-        raise ValueError(f"rope scaling {kind!r} is not supported (known: 'llama3')")
+        raise ValueError(f"rope scaling {kind!r} is not supported (known: 'llama3', 'yarn')")
     factor = float(scaling["factor"])
     lo, hi = float(scaling["low_freq_factor"]), float(scaling["high_freq_factor"])
     orig = float(scaling["original_max_position_embeddings"])
@@ -38,6 +55,13 @@ def inverse_frequencies(rot: int, theta: float, scaling: Optional[Mapping] = Non
     smooth = (orig / wavelen - lo) / (hi - lo)
     blended = (1.0 - smooth) * inv / factor + smooth * inv
     return np.where(wavelen < orig / hi, inv, np.where(wavelen > orig / lo, inv / factor, blended))
+
+
+def table_magnitude(scaling: Optional[Mapping] = None) -> float:
+    """What the table's cosines and sines are multiplied with: 0.1 * ln(factor) + 1 under the "yarn" rule, else 1."""
+    if scaling and scaling.get("rope_type") == "yarn":
+        return 0.1 * math.log(float(scaling["factor"])) + 1.0
+    return 1.0
 
 
 _TABLES: dict = {}
@@ -52,7 +76,7 @@ def rotary_table(rot: int, theta: float, rt: Runtime, scaling: Optional[Mapping]
     if t is None:
         pos = np.arange(rt.max_positions, dtype=np.float64)[:, None]
         ang = pos * inverse_frequencies(int(rot), float(theta), scaling)[None, :]
-        table = np.stack([np.cos(ang), np.sin(ang)], axis=1).astype(np.float32)
+        table = (np.stack([np.cos(ang), np.sin(ang)], axis=1) * table_magnitude(scaling)).astype(np.float32)
         if len(_TABLES) >= 16:
             _TABLES.clear()
         t = _TABLES[key] = torch.from_numpy(table).to(rt.device).contiguous()
@@ -77,7 +101,7 @@ class RotaryEncoding(PositionEncoding):
         self.rt = rt
         pos = np.arange(rt.max_positions, dtype=np.float64)[:, None]
         ang = pos * self.inv_freq[None, :]
-        table = np.stack([np.cos(ang), np.sin(ang)], axis=1).astype(np.float32)  # [positions, 2, rot/2]
+        table = (np.stack([np.cos(ang), np.sin(ang)], axis=1) * table_magnitude(self.scaling)).astype(np.float32)  # [positions, 2, rot/2]
         self.cos_sin = torch.from_numpy(table).to(rt.device).contiguous()
 
     def fused(self):

@@ -7,6 +7,8 @@ An expert is a gated unit Wd a(Wg h, Wu h) with tensors "<prefix><i>.gate|up|dow
 outputs of the router stand for experts without tensors that return h itself.  `activation` "silu": a(g, u) =
 silu(g) * u; "clamped": g' * sigmoid(alpha g') * (u' + 1) with g' = min(g, limit), u' = clamp(u, -limit, limit).
 With `renormalize` and no correction the weights are the softmax over the chosen logits alone.
+`score` "sigmoid": s = sigmoid(z), every expert for itself.  `weight_on` "input": the weight multiplies the expert's
+input instead of its output, out = sum of expert(weight * h).
 The choice is made on the GPU and stays there: nothing is read back, so steps replay in graphs."""
 from __future__ import annotations
 
@@ -25,7 +27,8 @@ class RoutedExperts(FeedForward):
 
     def __init__(self, hidden_size: int, intermediate_size: int, experts: int, top: int, identity: int = 0,
                  correction: bool = True, renormalize: bool = False, names: Optional[Mapping[str, str]] = None,
-                 activation: str = "silu", alpha: float = 1.0, limit: float = 0.0):
+                 activation: str = "silu", alpha: float = 1.0, limit: float = 0.0, score: str = "softmax",
+                 weight_on: str = "output"):
         self.D, self.F, self.E, self.K, self.I = (int(hidden_size), int(intermediate_size), int(experts), int(top),
                                                   int(identity))
         if self.E < 0 or self.I < 0 or not (1 <= self.K <= self.E + self.I):
@@ -35,6 +38,10 @@ class RoutedExperts(FeedForward):
             raise ValueError(f"routed experts: activation {activation!r} (known: {sorted(ops.EXPERT_ACTIVATIONS)}; "
                              f"the clamped unit needs a positive limit)")
         self.activation, self.alpha, self.limit = activation, float(alpha), float(limit)
+        if score not in ops.ROUTER_SCORES or weight_on not in ("output", "input"):
+            raise ValueError(f"routed experts: score {score!r} (known: {sorted(ops.ROUTER_SCORES)}), weight_on "
+                             f"{weight_on!r} ('output', 'input')")
+        self.score, self.weight_input = score, weight_on == "input"
         self.names = {"router": "router", "correction": "correction", "expert": "e", "gate": "gate", "up": "up",
                       "down": "down", **dict(names or {})}
 
@@ -76,8 +83,9 @@ class RoutedExperts(FeedForward):
         ops.linear(h, self.w_router, z)
         ids = torch.empty((T, self.K), dtype=torch.int32, device=dev)
         weights = torch.empty((T, self.K), dtype=torch.float32, device=dev)
-        ops.route_topk(z, self.correction_t, self.K, ids, weights, self.renormalize)
+        ops.route_topk(z, self.correction_t, self.K, ids, weights, self.renormalize, score=self.score)
         y = torch.empty((T, self.D), dtype=torch.float32, device=dev)
         ops.routed_experts(h, self.w_gate_up, self.w_down, self.E, self.F, ids, weights, self.K, y,
-                           activation=self.activation, alpha=self.alpha, limit=self.limit)
+                           activation=self.activation, alpha=self.alpha, limit=self.limit,
+                           weight_input=self.weight_input)
         return y

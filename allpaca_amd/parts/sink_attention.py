@@ -7,6 +7,9 @@
   s = (q . k) * scale over the keys the mask lets the row see ("causal": all earlier ones, "window": the last n)
   p = exp(s) / (exp(sink[head]) + sum exp(s)): the sink is a learned score a head, with no key and no value
   out = Wo (sum p v)
+Options: `qk_norm` (every q and k head is divided by its root mean square over the head and multiplied with the
+tensors "<q>.norm" / "<k>.norm" [key_dim], shared by all heads, before the rotation; values that are the keys stay as
+projected), `softcap` c (s <- c * tanh(s / c)), `rope_scaling` (a frequency rule of `parts/rope.py`).
 
 `latent_attention`: queries, keys and values go through low-rank latents.
   a = [Wdq; Wdkv; Wg] h                                   (one product; 32-bit rows)
@@ -40,7 +43,9 @@ class SinkAttention(Mixer):
 
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, key_dim: int, value_dim: int, scale: float,
                  rotary_dim: int = 0, rope_theta: float = 10000.0, mask: str = "causal", mask_size: int = 0,
-                 learned_sink: bool = True, values_are_keys: bool = False, names: Optional[Mapping[str, str]] = None):
+                 learned_sink: bool = True, values_are_keys: bool = False, names: Optional[Mapping[str, str]] = None,
+                 qk_norm: bool = False, norm_eps: float = 1e-6, softcap: float = 0.0,
+                 rope_scaling: Optional[Mapping] = None):
         if num_heads % num_kv_heads:
             raise ValueError(f"attention: {num_heads} heads are not a multiple of {num_kv_heads} kv heads")
         _check_mask(mask, mask_size)
@@ -54,7 +59,11 @@ class SinkAttention(Mixer):
         self.scale, self.theta = float(scale), float(rope_theta)
         self.mask, self.mask_size = mask, int(mask_size)
         self.learned_sink, self.values_are_keys = bool(learned_sink), bool(values_are_keys)
-        self.names = {"q": "q", "k": "k", "v": "v", "o": "o", "sink": "sink", **dict(names or {})}
+        self.qk_norm, self.eps, self.softcap = bool(qk_norm), float(norm_eps), float(softcap)
+        if self.softcap < 0:
+            raise ValueError(f"attention: the soft cap {softcap} must not be negative")
+        self.rope_scaling = dict(rope_scaling) if rope_scaling else None
+        self.names = {"q": "q", "k": "k", "v": "v", "o": "o", "sink": "sink", "norm": ".norm", **dict(names or {})}
         self.k_off = self.H * self.dk
         self.v_off = self.k_off if self.values_are_keys else self.k_off + self.G * self.dk
         self.width = self.k_off + self.G * self.dk + (0 if self.values_are_keys else self.G * self.dv)
@@ -66,6 +75,9 @@ class SinkAttention(Mixer):
             out[n["v"]] = ParamSpec((self.G * self.dv, self.D))
         if self.learned_sink:
             out[n["sink"]] = ParamSpec((self.H,), store="float32", init="normal")
+        if self.qk_norm:
+            out[n["q"] + n["norm"]] = ParamSpec((self.dk,), store="float32")
+            out[n["k"] + n["norm"]] = ParamSpec((self.dk,), store="float32")
         out[n["o"]] = ParamSpec((self.D, self.H * self.dv))
         return out
 
@@ -75,12 +87,16 @@ class SinkAttention(Mixer):
     def bind(self, tensors: Mapping[str, torch.Tensor], rt: Runtime) -> None:
         self.rt = rt
         n = self.names
+        self.q_norm_w = self.k_norm_w = None
+        if self.qk_norm:
+            self.q_norm_w = to_device(tensors[n["q"] + n["norm"]], rt, torch.float32)
+            self.k_norm_w = to_device(tensors[n["k"] + n["norm"]], rt, torch.float32)
         mats = [tensors[n["q"]], tensors[n["k"]]] + ([] if self.values_are_keys else [tensors[n["v"]]])
         dt = mats[0].dtype if all(m.dtype == mats[0].dtype for m in mats) else torch.float32
         self.w_in = ops.prepare_matrix(torch.cat([to_device(m, rt, dt) for m in mats], dim=0), rt.dtype)
         self.w_o = ops.prepare_matrix(to_device(tensors[n["o"]], rt), rt.dtype)
         self.sinks = to_device(tensors[n["sink"]], rt, torch.float32) if self.learned_sink else None
-        self.cos_sin = rotary_table(self.rot, self.theta, rt) if self.rot else None
+        self.cos_sin = rotary_table(self.rot, self.theta, rt, self.rope_scaling) if self.rot else None
 
     def forward(self, h, step, cache) -> torch.Tensor:
         """float32 [rows, hidden]: the mixer's output."""
@@ -94,10 +110,11 @@ class SinkAttention(Mixer):
         q = proj[:, :self.k_off]                    # rotated where it lies: a head is read whole before it is written
         ops.rotary_pages(proj, 0, self.H, self.dk, 0, q, proj, self.k_off, self.dk, None, 0, 0, False, 0,
                          proj, self.v_off, self.dv, self.G, self.rot, self.cos_sin, step, pages.block_table, pages.kv,
-                         pages.page_tokens)
+                         pages.page_tokens, q_norm_w=self.q_norm_w, k_norm_w=self.k_norm_w, norm_eps=self.eps)
         attn = torch.empty((T, self.H * self.dv), dtype=dt, device=dev)
         ops.masked_attention(q, attn, self.H, self.G, self.dk, self.dv, pages.kv, pages.page_tokens, pages.block_table,
-                             step, self.mask, self.mask_size, self.learned_sink, self.scale, sinks=self.sinks)
+                             step, self.mask, self.mask_size, self.learned_sink, self.scale, sinks=self.sinks,
+                             softcap=self.softcap)
         out = torch.empty((T, self.D), dtype=torch.float32, device=dev)
         ops.linear(attn, self.w_o, out)
         return out
