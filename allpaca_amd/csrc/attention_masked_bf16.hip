@@ -10,6 +10,10 @@
 // one head).  The kernels keep the whole key as the summed axis and give a head's query zeros outside its own part, so
 // nothing else changes; `out_f32`: the heads' outputs leave in float32 (for a caller that combines the maps).
 //
+// `softcap` c > 0: s <- c * tanh(s / c).  `r1`, `r2` [H]: s <- s - r1[h] * ln(1 + r2[h] * (p - t)) for the key at
+// position t, a learned penalty on the distance (behind the cap).  Both are applied to the float32 scores where they
+// leave the first product, ahead of the maximum; a launch without them runs as before.
+//
 // Pages: one row per kv head, first the page's keys [slot][dk], then its values [dv][slot]; a page is
 // G * P * (dk + dv) elements.
 //
@@ -54,6 +58,12 @@ __device__ __forceinline__ void keep_positions(Frag& v, int lo, int hi) {
   }
 }
 __device__ __forceinline__ float exp2_neg(float x) { return __builtin_amdgcn_exp2f(x); }
+// a scaled score through the soft cap and the distance penalty (d: how far back the key lies, not negative)
+__device__ __forceinline__ float shape_score(float x, float cap, bool penalty, float r1, float r2, int d) {
+  if (cap > 0.f) x = cap * (1.0f - 2.0f / (__expf(2.0f * x / cap) + 1.0f));
+  if (penalty) x -= r1 * __logf(1.0f + r2 * (float)d);
+  return x;
+}
 
 // ------------------------------------------------------------------------------------------ prompt portions
 template <int DKP, int DVP>  // key and value sizes rounded up to a multiple of 32
@@ -62,7 +72,8 @@ __global__ __launch_bounds__(256) void attn_masked_prefill_kernel(
     const bf16_t* __restrict__ cache, int P, const int* __restrict__ block_table, int max_blocks,
     const int* __restrict__ positions, const int* __restrict__ row_seg, const int* __restrict__ tile_row0,
     const int* __restrict__ tile_rows, int n_tiles, int mask, int mask_size, int sink, const float* __restrict__ sinks,
-    const float* __restrict__ gate, int ldg, float scale, int key_parts, int out_f32) {
+    const float* __restrict__ gate, int ldg, float scale, int key_parts, int out_f32, float softcap,
+    const float* __restrict__ r1, const float* __restrict__ r2) {
   constexpr int KROW = DKP + (DKP % 128 == 0 ? 72 : DKP % 128 == 64 ? 8 : DKP % 128 == 32 ? 40 : 104);
   __shared__ __attribute__((aligned(16))) bf16_t Ks[KT * KROW];
   __shared__ __attribute__((aligned(16))) bf16_t Vs[DVP * (KT + KPAD)];
@@ -113,7 +124,9 @@ __global__ __launch_bounds__(256) void attn_masked_prefill_kernel(
   const int my_lo = first_seen(my_pos, mask, mask_size);
   const int wave_hi = pos0 + wave * 16;                        // smallest position of the wave's rows
   const int wave_lo = first_seen(wave_hi + 15, mask, mask_size);  // largest first key of the wave's rows
-  const float sc2 = scale * LOG2E;
+  const bool shaped = softcap > 0.f || r1 != nullptr;       // scores are then finished (in base 2) before the maximum
+  const float r1h = r1 ? r1[h] : 0.f, r2h = r1 ? r2[h] : 0.f;
+  const float sc2 = shaped ? 1.f : scale * LOG2E;
   floatx4 o[DVP / 16];
 #pragma unroll
   for (int dt = 0; dt < DVP / 16; ++dt) o[dt] = floatx4{0.f, 0.f, 0.f, 0.f};
@@ -193,6 +206,15 @@ __global__ __launch_bounds__(256) void attn_masked_prefill_kernel(
         const Frag kf = *reinterpret_cast<const Frag*>(krd + nt * 16 * KROW + ks * 32);
         s[nt] = mfma16(kf, qf[ks], s[nt]);
       }
+    }
+    if (shaped) {
+#pragma unroll
+      for (int nt = 0; nt < KT / 16; ++nt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int d = my_pos - (t0 + nt * 16 + lc * 4 + r);
+          s[nt][r] = shape_score(s[nt][r] * scale, softcap, r1 != nullptr, r1h, r2h, d > 0 ? d : 0) * LOG2E;
+        }
     }
     float mx = -INFINITY;
     if (t0 >= wave_lo && t0 + KT - 1 <= wave_hi) {
@@ -294,7 +316,8 @@ __global__ __launch_bounds__(DT) void attn_masked_decode_kernel(
     const bf16_t* __restrict__ q, int ldq, int H, int G, int dk, int dv, const bf16_t* __restrict__ cache, int P,
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ positions,
     const int* __restrict__ row_seg, const int* __restrict__ rows, int mask, int mask_size, float scale, int n_splits,
-    float* __restrict__ parts, int key_parts) {
+    float* __restrict__ parts, int key_parts, float softcap, const float* __restrict__ r1,
+    const float* __restrict__ r2) {
   __shared__ __attribute__((aligned(16))) float sc_all[NW][HGMAX * SROW];
   __shared__ __attribute__((aligned(16))) bf16_t ps_all[NW][HGMAX * PROW];
   __shared__ float ml_all[NW][HGMAX][3];        // running maximum, running sum, the last pass's factor
@@ -322,6 +345,8 @@ __global__ __launch_bounds__(DT) void attn_masked_decode_kernel(
     qf[ks] = (li < per && c >= part0 && c < part0 + dq)
                  ? load_frag(q + (size_t)r * ldq + (size_t)(g * per + li) * dq + (c - part0)) : zero_frag();
   }
+  const bool shaped = softcap > 0.f || r1 != nullptr;
+  const float r1h = (r1 && li < per) ? r1[g * per + li] : 0.f, r2h = (r1 && li < per) ? r2[g * per + li] : 0.f;
   for (int idx = lane; idx < HGMAX * PROW; idx += WAVE) ps[idx] = 0;    // rows of heads that do not exist stay 0
   if (lane < HGMAX) { ml[lane][0] = -INFINITY; ml[lane][1] = 0.f; ml[lane][2] = 1.f; }
   floatx4 o[ET];
@@ -357,8 +382,15 @@ __global__ __launch_bounds__(DT) void attn_masked_decode_kernel(
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) acc = mfma16(kf[tt][ks], qf[ks], acc);
         // lane: keys tt * 16 + lc * 4 + 0..3 of the 64, head li
-        *reinterpret_cast<float4*>(sc + li * SROW + tt * 16 + lc * 4) =
-            float4{acc[0] * scale, acc[1] * scale, acc[2] * scale, acc[3] * scale};
+        float4 sv = float4{acc[0] * scale, acc[1] * scale, acc[2] * scale, acc[3] * scale};
+        if (shaped) {
+          const int d0 = pos - (t0 + tt * 16 + lc * 4);       // how far back the first of the four keys lies
+          sv.x = shape_score(sv.x, softcap, r1 != nullptr, r1h, r2h, d0 > 0 ? d0 : 0);
+          sv.y = shape_score(sv.y, softcap, r1 != nullptr, r1h, r2h, d0 > 1 ? d0 - 1 : 0);
+          sv.z = shape_score(sv.z, softcap, r1 != nullptr, r1h, r2h, d0 > 2 ? d0 - 2 : 0);
+          sv.w = shape_score(sv.w, softcap, r1 != nullptr, r1h, r2h, d0 > 3 ? d0 - 3 : 0);
+        }
+        *reinterpret_cast<float4*>(sc + li * SROW + tt * 16 + lc * 4) = sv;
       }
     }
     // ---- the value pieces are asked for now: they do not wait for the weights
@@ -503,10 +535,10 @@ APC_EXPORT int apc_attention_masked_prefill_bf16(const void* q, int ldq, void* o
                                                  int max_blocks, const int* positions, const int* row_seg,
                                                  const int* tile_row0, const int* tile_rows, int n_tiles, int mask,
                                                  int mask_size, int sink, const float* sinks, const float* gate,
-                                                 int ldg, float scale, int key_parts, int out_f32,
-                                                 hipStream_t stream) {
+                                                 int ldg, float scale, int key_parts, int out_f32, float softcap,
+                                                 const float* r1, const float* r2, hipStream_t stream) {
   if (n_tiles <= 0) return 0;
-  if ((sinks && !sink) || (gate && ldg < H)) return APC_ERR_BAD_ARG;
+  if ((sinks && !sink) || (gate && ldg < H) || softcap < 0.f || (!r1) != (!r2)) return APC_ERR_BAD_ARG;
   int e = check_sizes(q, ldq, out, ldo, cache, H, G, dk, dv, page_tokens, mask, mask_size, scale, key_parts, out_f32);
   if (e) return e;
   n_tiles *= 2;  // halves
@@ -516,7 +548,7 @@ APC_EXPORT int apc_attention_masked_prefill_bf16(const void* q, int ldq, void* o
   hipLaunchKernelGGL((attn_masked_prefill_kernel<DK_, DV_>), grid, block, 0, stream, (const bf16_t*)q, ldq,          \
                      out, ldo, H, G, dk, dv, (const bf16_t*)cache, page_tokens, block_table, max_blocks,             \
                      positions, row_seg, tile_row0, tile_rows, n_tiles, mask, mask_size, sink, sinks, gate, ldg,     \
-                     scale, key_parts, out_f32)
+                     scale, key_parts, out_f32, softcap, r1, r2)
 #define MP_VALUES(DK_)                       \
   do {                                       \
     if (dv <= 64) MP_LAUNCH(DK_, 64);        \
@@ -539,9 +571,10 @@ APC_EXPORT int apc_attention_masked_decode_bf16(const void* q, int ldq, void* ou
                                                 const int* row_seg, const int* rows, int mask, int mask_size, int sink,
                                                 const float* sinks, const float* gate, int ldg, float scale,
                                                 int n_splits, float* parts, int key_parts, int out_f32,
+                                                float softcap, const float* r1, const float* r2,
                                                 hipStream_t stream) {
   if (n_rows <= 0) return 0;
-  if ((sinks && !sink) || (gate && ldg < H)) return APC_ERR_BAD_ARG;
+  if ((sinks && !sink) || (gate && ldg < H) || softcap < 0.f || (!r1) != (!r2)) return APC_ERR_BAD_ARG;
   int e = check_sizes(q, ldq, out, ldo, cache, H, G, dk, dv, page_tokens, mask, mask_size, scale, key_parts, out_f32);
   if (e) return e;
   if (!apc_attention_masked_takes(H, G, dk, dv, page_tokens, key_parts)) return APC_ERR_UNSUPPORTED;
@@ -552,7 +585,7 @@ APC_EXPORT int apc_attention_masked_decode_bf16(const void* q, int ldq, void* ou
 #define MD_LAUNCH(KS_, ET_)                                                                                       \
   hipLaunchKernelGGL((attn_masked_decode_kernel<KS_, ET_>), grid, block, 0, stream, (const bf16_t*)q, ldq, H, G, dk, \
                      dv, (const bf16_t*)cache, page_tokens, block_table, max_blocks, positions, row_seg, rows, mask,  \
-                     mask_size, scale, n_splits, parts, key_parts)
+                     mask_size, scale, n_splits, parts, key_parts, softcap, r1, r2)
 #define MD_VALUES(KS_)                     \
   do {                                     \
     if (dv <= 64) MD_LAUNCH(KS_, 4);       \

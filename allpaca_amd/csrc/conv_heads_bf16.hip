@@ -3,6 +3,9 @@
 // its channels in registers.  Sums of squares of the pieces go through LDS, so a head may be any multiple of 8 wide,
 // and so may the width the norm is taken over (`norm_dim`, which divides a head; the normed values are multiplied with
 // q_norm_w / k_norm_w [norm_dim] if given).
+// `norm_rows`: the norm is taken over all heads of q (of k) at once, with weights of the projection's size; the
+// pieces' sums of a row are added by one wave for q and one for k.  `qt_every` > 0: q of the row at position p is
+// multiplied by 1 + qt_coef * ln(floor((p + 1) / qt_every) + 1).
 // The row holds q heads, then k heads, then v heads.  The state of the convolution is moved on by the plain kernel,
 // or here (`fold_state`) in a step of few rows in which every segment is a single row (decoded tokens).
 #include "mfma.h"
@@ -26,9 +29,9 @@ __global__ __launch_bounds__(NT) void conv_heads_bf16_kernel(
     const float* __restrict__ conv_w, float* __restrict__ state, int fold_state, int width,
     const int* __restrict__ row_seg, const int* __restrict__ seg_row0, const int* __restrict__ slots,
     const int* __restrict__ positions, int unit_norm, float eps, int norm_dim, const float* __restrict__ q_norm_w,
-    const float* __restrict__ k_norm_w, bf16_t* __restrict__ q_out, int ldq,
+    const float* __restrict__ k_norm_w, int norm_rows, float qt_coef, int qt_every, bf16_t* __restrict__ q_out, int ldq,
     const int* __restrict__ block_table, int max_blocks, bf16_t* __restrict__ cache, int P) {
-  extern __shared__ float ssum[];            // [ROWS][pieces]
+  extern __shared__ float ssum[];            // [ROWS][pieces], then [ROWS][2] (the sums over all of q and all of k)
   constexpr int taps = TAPS;
   const int tid = threadIdx.x;
   const int pieces = width / 8;
@@ -145,6 +148,19 @@ __global__ __launch_bounds__(NT) void conv_heads_bf16_kernel(
   }
   __syncthreads();
   const int kq = H * dk, kk = (H + G) * dk;
+  float* totals = ssum + ROWS * pieces;
+  if (norm_rows) {
+    // wave w adds the pieces of (row, q or k) number w, w + waves, ..: an order that the sizes alone fix
+    const int lane = tid % WAVE;
+    for (int job = tid / WAVE; job < ROWS * 2; job += NT / WAVE) {
+      const int rr = job / 2, first = (job % 2) ? kq / 8 : 0, n = (job % 2) ? (kk - kq) / 8 : kq / 8;
+      float t = 0.f;
+      for (int i = lane; i < n; i += WAVE) t += ssum[rr * pieces + first + i];
+      t = wave_sum(t);
+      if (lane == 0) totals[job] = t;
+    }
+    __syncthreads();
+  }
 #pragma unroll
   for (int k = 0; k < PPT; ++k) {
     const int p = tid + NT * k;
@@ -154,7 +170,8 @@ __global__ __launch_bounds__(NT) void conv_heads_bf16_kernel(
     const int d = kind == 2 ? dv : dk;
     const int rel = c0 - (kind == 0 ? 0 : kind == 1 ? kq : kk);
     const int head = rel / d, off = rel % d;
-    const int noff = off % norm_dim;                 // the piece's place in the range its norm is taken over
+    // the piece's place in the range its norm is taken over (and in that range's weights)
+    const int noff = norm_rows ? rel : off % norm_dim;
     float nw[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) nw[e] = 1.f;
@@ -168,12 +185,16 @@ __global__ __launch_bounds__(NT) void conv_heads_bf16_kernel(
       const int r = r0 + rr;
       if (r >= n_rows) continue;
       float inv = 1.f;
-      if (unit_norm && kind != 2) {
+      if (unit_norm && kind != 2 && norm_rows) {
+        inv = 1.0f / sqrtf(totals[rr * 2 + kind] / (float)(kind == 0 ? kq : kk - kq) + eps);
+      } else if (unit_norm && kind != 2) {
         const float* sp = ssum + rr * pieces + (c0 - noff) / 8;
         float ss = 0.f;
         for (int i = 0; i < norm_dim / 8; ++i) ss += sp[i];
         inv = 1.0f / sqrtf(ss / (float)norm_dim + eps);
       }
+      if (kind == 0 && qt_every > 0)      // (behind the weights in the plain kernel; a product of three either way)
+        inv *= 1.0f + qt_coef * logf((float)((positions[r] + 1) / qt_every) + 1.0f);
       Frag o;
 #pragma unroll
       for (int wd = 0; wd < 4; ++wd)
@@ -208,8 +229,9 @@ APC_EXPORT int apc_conv_heads_bf16_takes(int ld, int width, int H, int G, int dk
 APC_EXPORT int apc_conv_heads_bf16(const void* proj, int ld, int n_rows, int H, int G, int dk, int dv, const float* bias,
                                    const float* conv_w, int taps, float* state, int fold_state, int width, const int* row_seg,
                                    const int* seg_row0, const int* slots, const int* positions, int unit_norm, float eps,
-                                   int norm_dim, const float* q_norm_w, const float* k_norm_w, void* q_out, int ldq, const int* block_table, int max_blocks, void* cache,
-                                   int page_tokens, hipStream_t stream) {
+                                   int norm_dim, const float* q_norm_w, const float* k_norm_w, int norm_rows,
+                                   float qt_coef, int qt_every, void* q_out, int ldq, const int* block_table,
+                                   int max_blocks, void* cache, int page_tokens, hipStream_t stream) {
   if (n_rows <= 0) return 0;
   if (!apc_conv_heads_bf16_takes(ld, width, H, G, dk, dv, taps, ldq)) return APC_ERR_UNSUPPORTED;
   if (((uintptr_t)proj & 15u) || ((uintptr_t)q_out & 15u) || ((uintptr_t)cache & 15u) || ((uintptr_t)state & 15u) ||
@@ -217,7 +239,7 @@ APC_EXPORT int apc_conv_heads_bf16(const void* proj, int ld, int n_rows, int H, 
     return APC_ERR_UNSUPPORTED;
   if (taps > 1 && (!conv_w || !state || !slots)) return APC_ERR_BAD_ARG;
   if (norm_dim <= 0) norm_dim = dk;
-  if (dk % norm_dim) return APC_ERR_BAD_ARG;
+  if (dk % norm_dim || qt_every < 0 || (norm_rows && (!unit_norm || norm_dim != dk))) return APC_ERR_BAD_ARG;
   if (norm_dim % 8 || ((uintptr_t)q_norm_w & 15u) || ((uintptr_t)k_norm_w & 15u)) return APC_ERR_UNSUPPORTED;
   if (!conv_w && taps != 1) return APC_ERR_BAD_ARG;
   if (G > 0 && (!cache || !block_table || page_tokens <= 0 || max_blocks <= 0)) return APC_ERR_BAD_ARG;
@@ -230,11 +252,11 @@ APC_EXPORT int apc_conv_heads_bf16(const void* proj, int ld, int n_rows, int H, 
   const bool few = n_rows <= 32 || fold_state;
   const int rows_a_block = few ? 1 : pieces <= 768 ? 8 : 4;
   dim3 grid((n_rows + rows_a_block - 1) / rows_a_block), block(nt);
-  const size_t lds = (size_t)rows_a_block * pieces * sizeof(float);
+  const size_t lds = (size_t)rows_a_block * (pieces + 2) * sizeof(float);
 #define CH_LAUNCH(NT_, PPT_, ROWS_, TAPS_)                                                                          \
   hipLaunchKernelGGL((conv_heads_bf16_kernel<NT_, PPT_, ROWS_, TAPS_>), grid, block, lds, stream,                   \
                      (const bf16_t*)proj, ld, n_rows, H, G, dk, dv, bias, conv_w, state, fold_state, width, row_seg, seg_row0,  \
-                     slots, positions, unit_norm, eps, norm_dim, q_norm_w, k_norm_w, (bf16_t*)q_out, ldq, block_table, max_blocks, (bf16_t*)cache, \
+                     slots, positions, unit_norm, eps, norm_dim, q_norm_w, k_norm_w, norm_rows, qt_coef, qt_every, (bf16_t*)q_out, ldq, block_table, max_blocks, (bf16_t*)cache, \
                      page_tokens)
 #define CH_TAPS(NT_, PPT_, ROWS_)                            \
   do {                                                       \

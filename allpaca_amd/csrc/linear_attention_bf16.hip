@@ -270,7 +270,68 @@ constexpr size_t lds_bytes() {
          (C + 1) * 4;
 }
 
+// q and k of every row rotated by the row's position where they lie, k multiplied by k_scale behind the rotation:
+// what the chunk kernels then read.  A thread takes 8 consecutive elements of a head; in the first half of the rotated
+// range it takes its partner piece (rot / 2 further on) too, reads both and writes both; the thread of a piece in the
+// second half does nothing.
+__global__ __launch_bounds__(256) void linear_rotate_kernel(bf16_t* __restrict__ proj, int ld, int q_off, int k_off,
+                                                            int H, int dk, int rot, const float* __restrict__ cos_sin,
+                                                            const int* __restrict__ positions, float k_scale) {
+  const int r = blockIdx.x, per = dk / 8, half = rot / 2;
+  const int item = blockIdx.y * 256 + threadIdx.x;
+  if (item >= 2 * H * per) return;
+  const bool is_k = item >= H * per;
+  const int it = is_k ? item - H * per : item, h = it / per, e = (it % per) * 8;
+  bf16_t* head = proj + (size_t)r * ld + (is_k ? k_off : q_off) + (size_t)h * dk;
+  const float sc = is_k ? k_scale : 1.f;
+  float x[8], y[8];
+  if (e >= rot) {
+    if (sc != 1.f) {
+      unpack8f(load_frag(head + e), x);
+      Frag f;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) f.w[i] = pack_bf16x2(x[2 * i] * sc, x[2 * i + 1] * sc);
+      *reinterpret_cast<Frag*>(head + e) = f;
+    }
+    return;
+  }
+  if (e >= half) return;
+  unpack8f(load_frag(head + e), x);
+  unpack8f(load_frag(head + e + half), y);
+  const float* cs = cos_sin + (size_t)positions[r] * rot;
+  Frag fa, fb;
+  float a[8], b[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const float c = cs[e + i], sn = cs[half + e + i];
+    a[i] = (x[i] * c - y[i] * sn) * sc;
+    b[i] = (y[i] * c + x[i] * sn) * sc;
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    fa.w[i] = pack_bf16x2(a[2 * i], a[2 * i + 1]);
+    fb.w[i] = pack_bf16x2(b[2 * i], b[2 * i + 1]);
+  }
+  *reinterpret_cast<Frag*>(head + e) = fa;
+  *reinterpret_cast<Frag*>(head + e + half) = fb;
+}
+
 }  // namespace
+
+// q and k heads of bfloat16 rows rotated (and k scaled) in place; rot a multiple of 16, dk and the offsets of 8.
+APC_EXPORT int apc_linear_rotate_bf16(void* proj, int ld, int q_off, int k_off, int H, int dk, int rot,
+                                      const float* cos_sin, const int* positions, float k_scale, int n_rows,
+                                      hipStream_t stream) {
+  if (n_rows <= 0 || (rot == 0 && k_scale == 1.f)) return 0;
+  if (H <= 0 || dk <= 0 || rot < 0 || rot > dk || (rot && (!cos_sin || !positions))) return APC_ERR_BAD_ARG;
+  if (dk % 8 || rot % 16 || ld % 8 || q_off % 8 || k_off % 8 || ((uintptr_t)proj & 15u)) return APC_ERR_UNSUPPORTED;
+  const int items = 2 * H * (dk / 8);
+  if (ceil_div(items, 256) > 65535) return APC_ERR_UNSUPPORTED;
+  hipLaunchKernelGGL(linear_rotate_kernel, dim3(n_rows, ceil_div(items, 256)), dim3(256), 0, stream, (bf16_t*)proj, ld,
+                     q_off, k_off, H, dk, rot, cos_sin, positions, k_scale);
+  APC_LAUNCH_CHECK();
+  return 0;
+}
 
 // 1 if the kernel takes these sizes, else 0 (the caller then runs the plain kernel)
 APC_EXPORT int apc_linear_attention_bf16_takes(int ld, int q_off, int k_off, int v_off, int H, int dk, int dv) {

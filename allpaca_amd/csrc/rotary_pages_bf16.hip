@@ -10,6 +10,10 @@
 // many rows the values go through rotary_pages_values_kernel instead (16 rows x 128 columns through LDS, 8 slots of a
 // column in one store).
 // The second part of a key (the part all heads share, or a head's own) may be float32 rows.
+//
+// With a norm on the heads (q_norm_w / k_norm_w: a head over its root mean square, times weights all heads share,
+// ahead of the rotation) a wave takes a whole head of one row, a lane a piece: the sum of squares is the wave's, a lane
+// reads its piece and its partner's and writes its own, after all lanes have read (rotary_pages_norm_bf16_kernel).
 #include "mfma.h"
 #include <math.h>
 
@@ -108,6 +112,72 @@ __global__ __launch_bounds__(256) void rotary_pages_bf16_kernel(
   }
 }
 
+// One wave a (row, head): heads 0 .. H-1 are query heads, H .. H+G-1 keys (and their values).  d <= 512.
+__global__ __launch_bounds__(256) void rotary_pages_norm_bf16_kernel(
+    const bf16_t* q, int ldq, int q_off, int H, int dq, int q_rot0, bf16_t* q_out, int ldqo,     // (q_out may be q)
+    const bf16_t* __restrict__ ka, int ldka, int ka_off, int dk, int k_rot0, const bf16_t* __restrict__ v, int ldv,
+    int v_off, int dv, int G, int rot, const float* __restrict__ cos_sin, const int* __restrict__ positions,
+    const int* __restrict__ row_seg, const int* __restrict__ block_table, int max_blocks, bf16_t* __restrict__ cache,
+    int P, int with_values, const float* __restrict__ q_norm_w, const float* __restrict__ k_norm_w, float eps) {
+  const int r = blockIdx.x, hh = blockIdx.y * 4 + threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+  if (hh >= H + G) return;
+  const bool is_q = hh < H;
+  const int g = hh - H;
+  const int d = is_q ? dq : dk, rot0 = is_q ? q_rot0 : k_rot0, half = rot / 2;
+  const bf16_t* src = is_q ? q + (size_t)r * ldq + q_off + (size_t)hh * dq : ka + (size_t)r * ldka + ka_off + (size_t)g * dk;
+  const float* nw = is_q ? q_norm_w : k_norm_w;
+  const int pos = positions[r];
+  const int e = lane * 8;
+  const bool on = e < d;
+  F8 x = F8{{0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f}}, y = x;
+  if (on) x = load8_bf16(src + e);
+  const int j = e - rot0;
+  const bool turn = on && j >= 0 && j < rot, first = j < half;
+  const int pe = first ? e + half : e - half;        // the partner piece
+  if (turn) y = load8_bf16(src + pe);
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) ss = fmaf(x.v[i], x.v[i], ss);
+  ss = wave_sum(ss);
+  if (nw) {
+    const float inv = 1.0f / sqrtf(ss / (float)d + eps);
+    if (on) {
+      const F8 w = load8_f32(nw + e);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) x.v[i] = (x.v[i] * inv) * w.v[i];
+    }
+    if (turn) {
+      const F8 w = load8_f32(nw + pe);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) y.v[i] = (y.v[i] * inv) * w.v[i];
+    }
+  }
+  if (turn) {
+    const int jj = first ? j : j - half;
+    const float* cs = cos_sin + (size_t)pos * rot;
+    const F8 c = load8_f32(cs + jj), sn = load8_f32(cs + half + jj);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) x.v[i] = first ? x.v[i] * c.v[i] - y.v[i] * sn.v[i] : x.v[i] * c.v[i] + y.v[i] * sn.v[i];
+  }
+  if (is_q) {
+    if (on) store8_bf16(q_out + (size_t)r * ldqo + (size_t)hh * dq + e, x);
+    return;
+  }
+  const size_t page = (size_t)block_table[(size_t)row_seg[r] * max_blocks + pos / P];
+  const int slot = pos % P;
+  bf16_t* head = cache + (page * G + g) * (size_t)P * (dk + dv);
+  if (on) store8_bf16(head + (size_t)slot * dk + e, x);
+  if (with_values && e < dv) {
+    const Frag f = load_frag(v + (size_t)r * ldv + v_off + (size_t)g * dv + e);
+    bf16_t* dst = head + (size_t)P * dk + (size_t)e * P + slot;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      dst[(size_t)(2 * i) * P] = (bf16_t)(f.w[i] & 0xffffu);
+      dst[(size_t)(2 * i + 1) * P] = (bf16_t)(f.w[i] >> 16);
+    }
+  }
+}
+
 // The values of 16 rows x 128 columns (kv head * dv + element) through LDS into the transposed value blocks: where 8
 // rows are 8 consecutive slots of one page that start at a multiple of 8, a column's 8 values leave as one 16-byte
 // store; else slot by slot.
@@ -180,7 +250,8 @@ APC_EXPORT int apc_rotary_pages_bf16(const void* q, int ldq, int q_off, int H, i
                                      int ldkb, int kb_off, int db, int kb_shared, int k_rot0, const void* v, int ldv,
                                      int v_off, int dv, int G, int rot, const float* cos_sin, const int* positions,
                                      const int* row_seg, const int* block_table, int max_blocks, void* cache,
-                                     int page_tokens, int n_rows, hipStream_t stream) {
+                                     int page_tokens, int n_rows, const float* q_norm_w, const float* k_norm_w,
+                                     float norm_eps, hipStream_t stream) {
   if (n_rows <= 0) return 0;
   if (H <= 0 || G <= 0 || rot < 0 || (rot && !cos_sin) || !positions || !row_seg || !block_table || !cache || !q ||
       !q_out || !ka || !v || (db && !kb) || q_rot0 < 0 || q_rot0 + rot > dq || k_rot0 < 0 || k_rot0 + rot > da + db ||
@@ -196,11 +267,23 @@ APC_EXPORT int apc_rotary_pages_bf16(const void* q, int ldq, int q_off, int H, i
   const bool apart = n_rows >= 2 * VR && page_tokens % 8 == 0 && ((long)G * dv + VC - 1) / VC <= 65535;
   const long items = (long)H * (dq / 8) + (long)G * ((da + db) / 8) + (apart ? 0 : (long)G * (dv / 8));
   if (items > 65535L * 256) return APC_ERR_UNSUPPORTED;
+  const bool normed = q_norm_w || k_norm_w;
+  if (normed && (db || dq > 512 || da > 512 || dv > 512 || (H + G + 3) / 4 > 65535 || !aligned16(q_norm_w) ||
+                 !aligned16(k_norm_w)))
+    return APC_ERR_UNSUPPORTED;
   if (apart) {
     hipLaunchKernelGGL(rotary_pages_values_kernel, dim3((n_rows + VR - 1) / VR, (unsigned)((G * dv + VC - 1) / VC)),
                        dim3(256), 0, stream, (const bf16_t*)v, ldv, v_off, da + db, dv, G, positions, row_seg,
                        block_table, max_blocks, (bf16_t*)cache, page_tokens, n_rows);
     APC_LAUNCH_CHECK();
+  }
+  if (normed) {
+    hipLaunchKernelGGL(rotary_pages_norm_bf16_kernel, dim3(n_rows, (unsigned)((H + G + 3) / 4)), dim3(256), 0, stream,
+                       (const bf16_t*)q, ldq, q_off, H, dq, q_rot0, (bf16_t*)q_out, ldqo, (const bf16_t*)ka, ldka,
+                       ka_off, da, k_rot0, (const bf16_t*)v, ldv, v_off, dv, G, rot, cos_sin, positions, row_seg,
+                       block_table, max_blocks, (bf16_t*)cache, page_tokens, apart ? 0 : 1, q_norm_w, k_norm_w, norm_eps);
+    APC_LAUNCH_CHECK();
+    return 0;
   }
   hipLaunchKernelGGL(rotary_pages_bf16_kernel, dim3(n_rows, (unsigned)((items + 255) / 256)), dim3(256), 0, stream,
                      (const bf16_t*)q, ldq, q_off, H, dq, q_rot0, (bf16_t*)q_out, ldqo, (const bf16_t*)ka, ldka, ka_off,

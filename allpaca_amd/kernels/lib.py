@@ -82,18 +82,19 @@ SIGNATURES: Dict[str, Dict[str, list]] = {
         "apc_attention_prefill_bf16": [P, I, I, P, I, I, I, I, P, I, P, I, P, P, P, P, I, I, I, F, I, I, P, P],
         "apc_attention_decode_bf16": [P, I, I, P, I, I, I, I, I, P, I, P, I, P, P, P, I, F, I, I, P, P, P],
         "apc_conv_heads_bf16_takes": [I, I, I, I, I, I, I, I],
-        "apc_conv_heads_bf16": [P, I, I, I, I, I, I, P, P, I, P, I, I, P, P, P, P, I, F, I, P, P, P, I, P, I, P, I, P],
+        "apc_conv_heads_bf16": [P, I, I, I, I, I, I, P, P, I, P, I, I, P, P, P, P, I, F, I, P, P, I, F, I, P, I, P, I, P, I, P],
         "apc_routed_bf16_takes": [I, I, I],
         "apc_routed_max_tiles": [I, I, I],
         "apc_routed_experts_bf16": [P, I, P, P, I, I, I, P, P, I, I, I, P, P, P, P, P, I, I, F, F, I, P],
         "apc_linear_attention_bf16_takes": [I, I, I, I, I, I, I],
+        "apc_linear_rotate_bf16": [P, I, I, I, I, I, I, P, P, F, I, P],
         "apc_linear_attention_bf16": [P, I, I, I, I, I, I, I, I, P, P, I, P, P, P, I, P, P, P, P, I, P],
         "apc_attention_masked_takes": [I, I, I, I, I, I],
-        "apc_attention_masked_prefill_bf16": [P, I, P, I, I, I, I, I, P, I, P, I, P, P, P, P, I, I, I, I, P, P, I, F, I, I, P],
-        "apc_attention_masked_decode_bf16": [P, I, P, I, I, I, I, I, I, P, I, P, I, P, P, P, I, I, I, P, P, I, F, I, P, I, I, P],
+        "apc_attention_masked_prefill_bf16": [P, I, P, I, I, I, I, I, P, I, P, I, P, P, P, P, I, I, I, I, P, P, I, F, I, I, F, P, P, P],
+        "apc_attention_masked_decode_bf16": [P, I, P, I, I, I, I, I, I, P, I, P, I, P, P, P, I, I, I, P, P, I, F, I, P, I, I, F, P, P, P],
         "apc_rotary_pages_bf16_takes": [I] * 16,
         "apc_rotary_pages_bf16": [P, I, I, I, I, I, P, I, P, I, I, I, P, I, I, I, I, I, I, P, I, I, I, I, I, P, P, P, P, I,
-                                  P, I, I, P],
+                                  P, I, I, P, P, F, P],
         "apc_attention_decode_last_fits": [I, I, I, I],
         "apc_attention_decode_whole_fits": [I, I, I],
         "apc_attention_prefill_tile_rows": [],

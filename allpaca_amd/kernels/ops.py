@@ -422,7 +422,6 @@ def conv_heads(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, n_heads: 
     S = step.n_segs
     L = _lib.load("plain")
     if (_tuned_ok(proj, q_out) and (cache is None or cache.dtype == torch.bfloat16) and q_off == 0
-            and not norm_rows and not q_temp_every
             and (G == 0 or (k_off == n_heads * key_dim and v_off == (n_heads + G) * key_dim))):
         LT = _lib.load("tuned")
         if (LT.apc_conv_heads_bf16_takes(ld, width, n_heads, G, key_dim, value_dim, taps, ldq) and nd % 8 == 0
@@ -439,7 +438,8 @@ def conv_heads(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, n_heads: 
                 state.data_ptr() if taps > 1 else 0, 1 if fold else 0, width, _i32(step.row_seg, T, "row_seg"),
                 _i32(step.seg_row0, S, "seg_row0"), _i32(slots, S, "slots") if taps > 1 else 0,
                 _i32(step.positions, T, "positions"), 1 if unit_norm else 0, float(eps), nd,
-                _f32(q_norm_w, nd, "q norm weight"), _f32(k_norm_w, nd, "k norm weight"), q_out.data_ptr(), ldq,
+                _f32(q_norm_w, nq, "q norm weight"), _f32(k_norm_w, nk, "k norm weight"), 1 if norm_rows else 0,
+                float(q_temp_coef), int(q_temp_every), q_out.data_ptr(), ldq,
                 block_table.data_ptr() if G else 0, max_blocks, cache.data_ptr() if G else 0, page_tokens, _stream()),
                 "conv_heads_bf16")
             if taps > 1 and not fold:
@@ -557,11 +557,11 @@ def rotary_pages(q: torch.Tensor, q_off: int, n_heads: int, q_dim: int, q_rot0: 
     _split_pages(cache, G, da + db, dv, page_tokens)
     _need(block_table.dim() == 2 and block_table.dtype == torch.int32 and block_table.is_contiguous(),
           "block table must be contiguous int32 [segments, blocks]")
-    if _tuned_ok(q, q_out, ka, v, cache) and q_norm_w is None and k_norm_w is None:
+    if _tuned_ok(q, q_out, ka, v, cache):
         from . import tuned
         if tuned.rotary_pages_bf16(q, ldq, q_off, H, dq, q_rot0, q_out, ldqo, ka, ldka, ka_off, da, kb, ldkb, kb_off,
                                    db, kb_shared, k_rot0, v, ldv, v_off, dv, G, rot, cos_sin, step, block_table, cache,
-                                   page_tokens):
+                                   page_tokens, q_norm_w, k_norm_w, norm_eps):
             return
     L = _lib.load("plain")
     _lib.check(L.apc_rotary_pages(
@@ -693,7 +693,7 @@ def linear_attention(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, n_h
     `out` float32 [rows, heads * value_dim].  `powers` (optional): `tuned.decay_powers` of the same decay, kept by the
     caller for the kernel that walks prompt portions in chunks.  `rot` > 0: the first rot elements of every q and k
     head are rotated by the row's position (pairs i, i + rot/2; cos_sin float32 [positions, 2, rot/2]); `k_scale`
-    multiplies k behind the rotation."""
+    multiplies k behind the rotation.  (A bfloat16 step of prompt portions rotates q and k of `proj` where they lie.)"""
     _gpu(proj, decay, state, slots, out, powers, cos_sin)
     rot = int(rot)
     _need(rot % 2 == 0 and 0 <= rot <= int(key_dim), "linear attention: the rotated width must be even and at most key_dim")
@@ -710,10 +710,10 @@ def linear_attention(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, n_h
     _need(state.dtype == torch.float32 and state.is_contiguous() and tuple(state.shape[1:]) == (H, dk, dv),
           f"linear attention: state must be float32 [slots, {H}, {dk}, {dv}]")
     S = step.n_segs
-    if _tuned_ok(proj) and not rot and float(k_scale) == 1.0:
+    if _tuned_ok(proj):
         from . import tuned
         if tuned.linear_attention_bf16(proj, q_off, k_off, v_off, H, dk, dv, silu, decay, state, step, slots, out,
-                                       powers):
+                                       powers, rot, cos_sin, k_scale):
             return
     L = _lib.load("plain")
     _lib.check(L.apc_linear_attention(proj.data_ptr(), _code(proj), ld, q_off, k_off, v_off, H, dk, dv,

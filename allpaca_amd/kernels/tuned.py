@@ -473,8 +473,8 @@ def masked_attention_bf16(q, out, n_heads, n_kv_heads, key_dim, value_dim, cache
     f32 = out.dtype == torch.float32
     if gate is not None and gate.dtype != torch.float32:
         return False
-    if softcap or distance_bias is not None:
-        return False
+    r1, r2 = distance_bias if distance_bias is not None else (None, None)
+    r1_p, r2_p = _ops._f32(r1, n_heads, "distance bias r1"), _ops._f32(r2, n_heads, "distance bias r2")
     _ops._check_sinks_gate(sink, sinks, gate, T, n_heads)
     sinks_p = _ops._f32(sinks, n_heads, "sinks")
     gate_p, ldg = (gate.data_ptr(), _ops._rows(gate, "head gate")) if gate is not None else (0, 0)
@@ -497,7 +497,7 @@ def masked_attention_bf16(q, out, n_heads, n_kv_heads, key_dim, value_dim, cache
             page_tokens, block_table.data_ptr(), block_table.shape[1], step.positions.data_ptr(),
             step.row_seg.data_ptr(), step.tile_row0.data_ptr(), step.tile_rows.data_ptr(), step.n_tiles, code,
             int(mask_size), 1 if sink else 0, sinks_p, gate_p, ldg, float(scale), int(key_parts), 1 if f32 else 0,
-            stream), "attention_masked_prefill_bf16")
+            float(softcap), r1_p, r2_p, stream), "attention_masked_prefill_bf16")
     if step.n_decode_rows:
         n = step.n_decode_rows
         keys = min(step.max_decode_context, mask_size) if code else step.max_decode_context
@@ -509,7 +509,7 @@ def masked_attention_bf16(q, out, n_heads, n_kv_heads, key_dim, value_dim, cache
             page_tokens, block_table.data_ptr(), block_table.shape[1], step.positions.data_ptr(),
             step.row_seg.data_ptr(), step.decode_rows.data_ptr() if step.decode_rows is not None else 0, code,
             int(mask_size), 1 if sink else 0, sinks_p, gate_p, ldg, float(scale), splits, parts.data_ptr(),
-            int(key_parts), 1 if f32 else 0, stream), "attention_masked_decode_bf16")
+            int(key_parts), 1 if f32 else 0, float(softcap), r1_p, r2_p, stream), "attention_masked_decode_bf16")
     return True
 
 
@@ -517,15 +517,24 @@ LINEAR_CHUNK_MIN_ROWS = 5    # segments of at least this many rows make a step r
 
 
 def linear_attention_bf16(proj, q_off, k_off, v_off, H, dk, dv, silu, decay, state, step, slots, out,
-                          powers=None) -> bool:
+                          powers=None, rot: int = 0, cos_sin=None, k_scale: float = 1.0) -> bool:
     """Linear attention with a decay on the MFMA kernel that walks a segment in chunks of 64 rows.  False (nothing
     done) for sizes it does not take and for steps whose segments are all short (decoded rows): the caller then runs
-    the kernel that walks row by row."""
+    the kernel that walks row by row.  With a rotation or a key scale, q and k of `proj` are first rotated (and k
+    scaled) where they lie, in bfloat16: the chunk kernels' operands are 16 bits anyway."""
     ld, ldo = _ops._rows(proj, "projected rows"), _ops._rows(out, "linear attention out")
     L = _lib.load("tuned")
     if (step.max_rows < LINEAR_CHUNK_MIN_ROWS or proj.dtype != torch.bfloat16 or ldo % 4 or not _aligned(proj, out)
             or not L.apc_linear_attention_bf16_takes(ld, q_off, k_off, v_off, H, dk, dv)):
         return False
+    if rot or float(k_scale) != 1.0:
+        if silu or rot % 16 or (rot and not _aligned(cos_sin)):
+            return False
+        T = proj.shape[0]
+        _lib.check(L.apc_linear_rotate_bf16(proj.data_ptr(), ld, q_off, k_off, H, dk, int(rot),
+                                            cos_sin.data_ptr() if rot else 0,
+                                            _ops._i32(step.positions, T, "positions") if rot else 0, float(k_scale), T,
+                                            _ops._stream()), "linear_rotate_bf16")
     S = step.n_segs
     if powers is None:         # (a caller that keeps the table, as the mixer does, saves this read-back)
         powers = decay_powers(decay.tolist(), proj.device)
@@ -620,7 +629,8 @@ def routed_experts_bf16(h, w_gate_up: PackedExperts, w_down: PackedExperts, E: i
 
 
 def rotary_pages_bf16(q, ldq, q_off, H, dq, q_rot0, q_out, ldqo, ka, ldka, ka_off, da, kb, ldkb, kb_off, db, kb_shared,
-                      k_rot0, v, ldv, v_off, dv, G, rot, cos_sin, step, block_table, cache, page_tokens) -> bool:
+                      k_rot0, v, ldv, v_off, dv, G, rot, cos_sin, step, block_table, cache, page_tokens, q_norm_w=None,
+                      k_norm_w=None, norm_eps: float = 0.0) -> bool:
     """Heads put together, rotated and written into the pages on 16-byte accesses (bfloat16 rows and pages; the second
     key part may be float32 rows); False (nothing done) for sizes the kernel does not take."""
     L = _lib.load("tuned")
@@ -632,10 +642,15 @@ def rotary_pages_bf16(q, ldq, q_off, H, dq, q_rot0, q_out, ldqo, ka, ldka, ka_of
         return False
     if not _aligned(q, q_out, ka, v, cache) or (kb is not None and not _aligned(kb)) or (rot and not _aligned(cos_sin)):
         return False
+    if q_norm_w is not None or k_norm_w is not None:
+        # a wave a head: no second key part, heads of up to 512 elements
+        if kb is not None or db or max(dq, da, dv) > 512 or not all(w is None or _aligned(w) for w in (q_norm_w, k_norm_w)):
+            return False
     _lib.check(L.apc_rotary_pages_bf16(
         q.data_ptr(), ldq, q_off, H, dq, q_rot0, q_out.data_ptr(), ldqo, ka.data_ptr(), ldka, ka_off, da,
         kb.data_ptr() if kb is not None else 0, 1 if kb is not None and kb.dtype == torch.float32 else 0, ldkb, kb_off,
         db, 1 if kb_shared else 0, k_rot0, v.data_ptr(), ldv, v_off, dv, G, rot, cos_sin.data_ptr() if rot else 0,
         _ops._i32(step.positions, T, "positions"), _ops._i32(step.row_seg, T, "row_seg"), block_table.data_ptr(),
-        block_table.shape[1], cache.data_ptr(), page_tokens, T, _ops._stream()), "rotary_pages_bf16")
+        block_table.shape[1], cache.data_ptr(), page_tokens, T, _ops._f32(q_norm_w, dq, "q norm weight"),
+        _ops._f32(k_norm_w, da + db, "k norm weight"), float(norm_eps), _ops._stream()), "rotary_pages_bf16")
     return True
