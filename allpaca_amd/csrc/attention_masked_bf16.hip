@@ -58,11 +58,32 @@ __device__ __forceinline__ void keep_positions(Frag& v, int lo, int hi) {
   }
 }
 __device__ __forceinline__ float exp2_neg(float x) { return __builtin_amdgcn_exp2f(x); }
-// a scaled score through the soft cap and the distance penalty (d: how far back the key lies, not negative)
-__device__ __forceinline__ float shape_score(float x, float cap, bool penalty, float r1, float r2, int d) {
-  if (cap > 0.f) x = cap * (1.0f - 2.0f / (__expf(2.0f * x / cap) + 1.0f));
-  if (penalty) x -= r1 * __logf(1.0f + r2 * (float)d);
-  return x;
+// A product q . k through the scale, the soft cap and the distance penalty, in units of `unit` (1: natural, log2(e):
+// the exponent's base 2), with the constants folded by the caller:
+//   no cap:  dot * mul;                      mul = scale * unit
+//   cap c:   out * tanh(dot * scale / c) = out * (1 - 2 / (2^(dot * in) + 1));   in = 2 log2(e) scale / c, out = c * unit
+//   penalty: less pen * log2(1 + r2 * d);    pen = r1 * ln 2 * unit  (d: how far back the key lies, not negative)
+struct ScoreShape {
+  float mul, in, out, pen, r2;
+  bool capped, penalty;
+};
+__device__ __forceinline__ ScoreShape score_shape(float scale, float cap, const float* r1, const float* r2, int head,
+                                                  float unit) {
+  ScoreShape f;
+  f.capped = cap > 0.f;
+  f.penalty = r1 != nullptr;
+  f.mul = scale * unit;
+  f.in = f.capped ? 2.0f * LOG2E * scale / cap : 0.f;
+  f.out = cap * unit;
+  f.pen = f.penalty ? r1[head] * 0.6931471805599453f * unit : 0.f;
+  f.r2 = f.penalty ? r2[head] : 0.f;
+  return f;
+}
+__device__ __forceinline__ float shape_score(float dot, const ScoreShape& f, int d) {
+  float v = dot * f.mul;
+  if (f.capped) v = f.out * (1.0f - 2.0f * __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(dot * f.in) + 1.0f));
+  if (f.penalty) v = fmaf(-f.pen, __log2f(fmaf(f.r2, (float)d, 1.0f)), v);
+  return v;
 }
 
 // ------------------------------------------------------------------------------------------ prompt portions
@@ -125,7 +146,7 @@ __global__ __launch_bounds__(256) void attn_masked_prefill_kernel(
   const int wave_hi = pos0 + wave * 16;                        // smallest position of the wave's rows
   const int wave_lo = first_seen(wave_hi + 15, mask, mask_size);  // largest first key of the wave's rows
   const bool shaped = softcap > 0.f || r1 != nullptr;       // scores are then finished (in base 2) before the maximum
-  const float r1h = r1 ? r1[h] : 0.f, r2h = r1 ? r2[h] : 0.f;
+  const ScoreShape shape = score_shape(scale, softcap, r1, r2, h, LOG2E);
   const float sc2 = shaped ? 1.f : scale * LOG2E;
   floatx4 o[DVP / 16];
 #pragma unroll
@@ -213,7 +234,7 @@ __global__ __launch_bounds__(256) void attn_masked_prefill_kernel(
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           const int d = my_pos - (t0 + nt * 16 + lc * 4 + r);
-          s[nt][r] = shape_score(s[nt][r] * scale, softcap, r1 != nullptr, r1h, r2h, d > 0 ? d : 0) * LOG2E;
+          s[nt][r] = shape_score(s[nt][r], shape, d > 0 ? d : 0);
         }
     }
     float mx = -INFINITY;
@@ -346,7 +367,7 @@ __global__ __launch_bounds__(DT) void attn_masked_decode_kernel(
                  ? load_frag(q + (size_t)r * ldq + (size_t)(g * per + li) * dq + (c - part0)) : zero_frag();
   }
   const bool shaped = softcap > 0.f || r1 != nullptr;
-  const float r1h = (r1 && li < per) ? r1[g * per + li] : 0.f, r2h = (r1 && li < per) ? r2[g * per + li] : 0.f;
+  const ScoreShape shape = score_shape(scale, softcap, r1, r2, g * per + (li < per ? li : 0), 1.0f);
   for (int idx = lane; idx < HGMAX * PROW; idx += WAVE) ps[idx] = 0;    // rows of heads that do not exist stay 0
   if (lane < HGMAX) { ml[lane][0] = -INFINITY; ml[lane][1] = 0.f; ml[lane][2] = 1.f; }
   floatx4 o[ET];
@@ -385,10 +406,10 @@ __global__ __launch_bounds__(DT) void attn_masked_decode_kernel(
         float4 sv = float4{acc[0] * scale, acc[1] * scale, acc[2] * scale, acc[3] * scale};
         if (shaped) {
           const int d0 = pos - (t0 + tt * 16 + lc * 4);       // how far back the first of the four keys lies
-          sv.x = shape_score(sv.x, softcap, r1 != nullptr, r1h, r2h, d0 > 0 ? d0 : 0);
-          sv.y = shape_score(sv.y, softcap, r1 != nullptr, r1h, r2h, d0 > 1 ? d0 - 1 : 0);
-          sv.z = shape_score(sv.z, softcap, r1 != nullptr, r1h, r2h, d0 > 2 ? d0 - 2 : 0);
-          sv.w = shape_score(sv.w, softcap, r1 != nullptr, r1h, r2h, d0 > 3 ? d0 - 3 : 0);
+          sv.x = shape_score(acc[0], shape, d0 > 0 ? d0 : 0);
+          sv.y = shape_score(acc[1], shape, d0 > 1 ? d0 - 1 : 0);
+          sv.z = shape_score(acc[2], shape, d0 > 2 ? d0 - 2 : 0);
+          sv.w = shape_score(acc[3], shape, d0 > 3 ? d0 - 3 : 0);
         }
         *reinterpret_cast<float4*>(sc + li * SROW + tt * 16 + lc * 4) = sv;
       }

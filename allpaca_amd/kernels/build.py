@@ -26,7 +26,7 @@ LIBS: Dict[str, List[str]] = {
     "plain": ["plain_ops.hip", "plain_gemm.hip", "plain_attention.hip", "plain_mixers.hip", "plain_heads.hip", "plain_recurrent.hip", "plain_routed.hip",
               "plain_scan.hip", "sampling.hip"],
     "tuned": ["gemm_bf16.hip", "gemm_wide_bf16.hip", "gemm_direct_bf16.hip", "skinny_gemm_bf16.hip", "attention_bf16.hip", "attention_wide_bf16.hip", "attention_masked_bf16.hip", "conv_heads_bf16.hip", "rope_bf16.hip", "rotary_pages_bf16.hip",
-              "linear_attention_bf16.hip", "routed_bf16.hip"],
+              "linear_attention_bf16.hip", "routed_bf16.hip", "selective_scan_bf16.hip"],
     # what measurements need and the engine does not (what a streaming read and a loop of MFMAs reach on this card)
     "bench": ["probe.hip"],
     "host": ["host/exec.cpp", "host/cache.cpp", "host/pack.cpp", "host/sched.cpp"],

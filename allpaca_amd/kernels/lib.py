@@ -87,6 +87,8 @@ SIGNATURES: Dict[str, Dict[str, list]] = {
         "apc_routed_max_tiles": [I, I, I],
         "apc_routed_experts_bf16": [P, I, P, P, I, I, I, P, P, I, I, I, P, P, P, P, P, I, I, F, F, I, P],
         "apc_linear_attention_bf16_takes": [I, I, I, I, I, I, I],
+        "apc_selective_scan_bf16_takes": [I, I],
+        "apc_selective_scan_bf16": [P, I, P, I, P, P, P, I, P, P, I, P, I, I, I, P, P, P, I, P, P, P, P, P, I, P],
         "apc_linear_rotate_bf16": [P, I, I, I, I, I, I, P, P, F, I, P],
         "apc_linear_attention_bf16": [P, I, I, I, I, I, I, I, I, P, P, I, P, P, P, I, P, P, P, P, I, P],
         "apc_attention_masked_takes": [I, I, I, I, I, I],
@@ -141,7 +143,7 @@ class KernelTimer:
 
 _timer = None
 # entry points that launch nothing (questions about sizes): never timed
-NOT_KERNELS = {"apc_attention_masked_takes", "apc_rotary_pages_bf16_takes", "apc_routed_bf16_takes", "apc_routed_max_tiles", "apc_linear_attention_bf16_takes", "apc_conv_heads_bf16_takes", "apc_attention_decode_whole_fits", "apc_attention_decode_last_fits", "apc_attention_prefill_tile_rows",
+NOT_KERNELS = {"apc_selective_scan_bf16_takes", "apc_attention_masked_takes", "apc_rotary_pages_bf16_takes", "apc_routed_bf16_takes", "apc_routed_max_tiles", "apc_linear_attention_bf16_takes", "apc_conv_heads_bf16_takes", "apc_attention_decode_whole_fits", "apc_attention_decode_last_fits", "apc_attention_prefill_tile_rows",
                "apc_attention_prefill_wide_takes",
                "apc_gemm_direct_k_split", "apc_gemm_direct_emit_parts", "apc_sample_rows_scratch_kib"}
 

@@ -883,6 +883,10 @@ def selective_scan(x: torch.Tensor, dt: torch.Tensor, dt_bias: Optional[torch.Te
     _need(state.dtype == torch.float32 and state.is_contiguous() and tuple(state.shape[1:]) == (C, N),
           f"selective_scan: state must be float32 [slots, {C}, {N}]")
     S = step.n_segs
+    if _tuned_ok(x, z, out):
+        from . import tuned
+        if tuned.selective_scan_bf16(x, dt, dt_bias, A, bc, D, z, state, step, slots, out):
+            return
     L = _lib.load("plain")
     _lib.check(L.apc_selective_scan(x.data_ptr(), _code(x), _rows(x, "x"), dt.data_ptr(), _rows(dt, "dt"),
                                     _f32(dt_bias, C, "dt bias"), A.data_ptr(), bc.data_ptr(), _rows(bc, "B and C"),

@@ -549,6 +549,31 @@ def linear_attention_bf16(proj, q_off, k_off, v_off, H, dk, dv, silu, decay, sta
     return True
 
 
+SCAN_CHUNK_MIN_ROWS = 5      # as above, for the selective scan
+
+
+def selective_scan_bf16(x, dt, dt_bias, A, bc, D, z, state, step, slots, out) -> bool:
+    """The selective scan over prompt portions, chunks of 64 rows side by side (summaries, a scan over the chunks, the
+    outputs).  False (nothing done) for sizes the kernels do not take and for steps whose segments are all short
+    (decoded rows): the caller then runs the kernel that walks row by row."""
+    L = _lib.load("tuned")
+    T, C = out.shape
+    N = int(A.shape[1])
+    if step.max_rows < SCAN_CHUNK_MIN_ROWS or not L.apc_selective_scan_bf16_takes(C, N):
+        return False
+    S = step.n_segs
+    n_chunks, chunks, seg_chunks = _row_chunks(step, x.device)
+    ws = torch.empty((n_chunks, C, N), dtype=torch.float32, device=x.device)
+    sums = torch.empty((n_chunks, C), dtype=torch.float32, device=x.device)
+    _lib.check(L.apc_selective_scan_bf16(
+        x.data_ptr(), _ops._rows(x, "x"), dt.data_ptr(), _ops._rows(dt, "dt"), _ops._f32(dt_bias, C, "dt bias"),
+        A.data_ptr(), bc.data_ptr(), _ops._rows(bc, "B and C"), _ops._f32(D, C, "D"), z.data_ptr(), _ops._rows(z, "z"),
+        state.data_ptr(), C, N, S, _ops._i32(step.seg_row0, S, "seg_row0"), _ops._i32(step.seg_rows, S, "seg_rows"),
+        _ops._i32(slots, S, "slots"), n_chunks, chunks.data_ptr(), seg_chunks.data_ptr(), ws.data_ptr(),
+        sums.data_ptr(), out.data_ptr(), _ops._rows(out, "out"), _ops._stream()), "selective_scan_bf16")
+    return True
+
+
 LINEAR_CHUNK_ROWS = 64
 
 

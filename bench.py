@@ -681,6 +681,141 @@ def lesarax_run(args) -> int:
     return 0
 
 
+# ---- the Seredra design beside the llama decoder at equal sizes ---------------------------------------------------
+SEREDRA_LIKE_KERNELS = {
+    "apc_conv_heads_bf16": ["apc_rope_kv_write_bf16", "apc_rope_kv_write"],
+    "apc_rotary_pages_bf16": ["apc_rope_kv_write_bf16", "apc_rope_kv_write"],
+    "apc_attention_masked_prefill_bf16": ["apc_attention_prefill_bf16"],
+    "apc_attention_masked_decode_bf16": ["apc_attention_decode_bf16"],
+    "apc_linear_attention_bf16": ["apc_attention_prefill_bf16"],
+    "apc_linear_attention": ["apc_attention_decode_bf16"],
+    "apc_selective_scan": ["apc_attention_prefill_bf16", "apc_attention_decode_bf16"],
+    "apc_conv_channels": ["apc_rope_kv_write_bf16", "apc_rope_kv_write"],
+    "apc_routed_experts_bf16": ["apc_gemm_swiglu_bf16", "apc_skinny_swiglu_bf16", "apc_skinny_swiglu_pre_bf16"],
+    "apc_act_rows": [],
+    "apc_streams_step": ["apc_rmsnorm_rows"],
+    "apc_gated_rmsnorm": [],
+    "apc_weighted_pair": [],
+}
+SEREDRA_EXPERTS, SEREDRA_TOP, SEREDRA_STATES, SEREDRA_TAPS = 8, 2, 16, 4
+
+
+def seredra_configs(size: str, context: int):
+    """Four layers: the convolution attention (4 taps, temperature, distance penalty) with the squared-relu
+    feed-forward; a retention (heads of d) with routed experts (2 of 8, each half as wide as the dense feed-forward: the
+    same arithmetic a row); the side-by-side mixer (grouped attention whose values are its keys, half of a head rotated
+    under the frequency rule, soft cap; a selective scan of 2 x width channels with 16 states) with the dense
+    feed-forward; an attention that borrows the first one's keys and values, with experts.  The llama decoder with four
+    layers of the same widths."""
+    D, H, G, d, F, V = DESIGN_SIZES[size]
+    att = dict(heads=H, kv_heads=G, dim=d, vdim=d, scale=d ** -0.5, conv=SEREDRA_TAPS, q_temp=dict(coef=0.1, every=256))
+    left = dict(heads=H, kv_heads=G, dim=d, vdim=d, scale=d ** -0.5, softcap=50.0,
+                rot=dict(base=500000.0, dims=d // 2, scaling=dict(factor=4.0, original=2048, fast=32.0, slow=1.0)))
+    right = dict(inner=2 * D, state=SEREDRA_STATES, dt_rank=D // 16, conv=SEREDRA_TAPS)
+    ret = dict(heads=H, dim=d, vdim=d, decay=[1.0 - 2.0 ** (-5 - 5 * h / H) for h in range(H)],
+               rot=dict(base=10000.0, dims=d))
+    moe = dict(kind="moe", expert=dict(ff=F // SEREDRA_TOP), router=dict(experts=SEREDRA_EXPERTS, top=SEREDRA_TOP))
+    dense = dict(kind="dense", ff=F)
+    seredra = dict(architecture="Seredra", vocab=V, width=D, embedding=dict(scale=1.0), norm=dict(eps=1e-6),
+                   max_positions=2 * context + 4096,
+                   layers=[dict(type="attention", mixer=att, mlp=dense),
+                           dict(type="retention", mixer=ret, mlp=moe),
+                           dict(type="parallel", mixer=dict(left=left, right=right, left_scale=0.7, right_scale=0.7),
+                                mlp=dense),
+                           dict(type="attention", mixer=dict(att, kv_from=0), mlp=moe)])
+    return {"seredra": seredra, "llama": design_configs(size, 4, 2 * context)["llama"]}
+
+
+def seredra_rooflines(size, batch, context, T, points):
+    """For the kernels the design adds and their like kernels of the llama decoder: the bytes or the arithmetic of the
+    launches of a step over the measured time, as a share of the GPU's peak (8 TB/s, 2.5 PFLOP/s)."""
+    D, H, G, d, F, V = DESIGN_SIZES[size]
+    Fe, E, K, N, C = F // SEREDRA_TOP, SEREDRA_EXPERTS, SEREDRA_TOP, SEREDRA_STATES, 2 * D
+
+    def work(name, rows, keys_sum, prefill):
+        """(bytes, flops) of all of a step's launches of entry point `name`."""
+        if name == "apc_conv_heads_bf16":        # an owner (q, k, v) and a borrower (q): rows read, q and pages written
+            return 2 * rows * ((H + 2 * G) * d + H * d) * 2 * 2 - 2 * rows * 2 * G * d * 2 * 2 // 2, 0
+        if name == "apc_rotary_pages_bf16":      # q and k read, q and the pages' keys and values written
+            return rows * ((H + G) * d + H * d + 2 * G * d) * 2, 0
+        if name in ("apc_rope_kv_write_bf16", "apc_rope_kv_write"):
+            return 4 * rows * ((H + 2 * G) * d + H * d + 2 * G * d) * 2, 0
+        if name == "apc_attention_masked_prefill_bf16":      # three attentions over all earlier keys
+            return 0, 3 * keys_sum * H * 4 * d
+        if name == "apc_attention_prefill_bf16":
+            return 0, 4 * 4 * keys_sum * H * d
+        if name == "apc_attention_masked_decode_bf16":
+            return 3 * keys_sum * G * 2 * d * 2, 0
+        if name == "apc_attention_decode_bf16":
+            return 4 * keys_sum * G * 2 * d * 2, 0
+        if name == "apc_linear_attention_bf16":  # a row: scores and weights over half a chunk of 64, 2 dk dv for the state
+            return 0, rows * H * (2 * 32 * 2 * d + 2 * 2 * d * d)
+        if name == "apc_linear_attention":       # the state of every row read and written
+            return rows * H * d * d * 4 * 2, 0
+        if name == "apc_selective_scan":         # x, z, the step sizes read, y written; decoded rows: the state both ways
+            return rows * C * (2 + 2 + 4 + 2) + (0 if prefill else rows * C * N * 4 * 2), 0
+        if name == "apc_conv_channels":
+            return rows * C * (2 + 2), 0
+        if name == "apc_routed_experts_bf16":
+            used = min(E, rows * K)
+            return 2 * used * 3 * Fe * D * 2, 2 * rows * K * 3 * 2 * Fe * D
+        if name in ("apc_gemm_swiglu_bf16", "apc_skinny_swiglu_bf16", "apc_skinny_swiglu_pre_bf16"):
+            return 4 * 2 * F * D * 2, 4 * rows * 2 * 2 * F * D
+        if name == "apc_act_rows":               # the float32 sums read, the activations written
+            return 2 * rows * F * (4 + 2), 0
+        if name == "apc_streams_step":           # y and x read, x and the next reader's 16-bit copy written
+            return 9 * rows * D * (4 + 4 + 4 + 2), 0
+        if name == "apc_rmsnorm_rows":
+            return 9 * rows * D * (4 + 2), 0
+        if name == "apc_gated_rmsnorm":
+            return rows * H * d * (4 + 2 + 2), 0
+        if name == "apc_weighted_pair":
+            return rows * D * 12, 0
+        return None
+
+    table = {}
+    for phase, rows, keys_sum in (("prefill", T, T * (T + 1) // 2), ("decode", batch, batch * context)):
+        for new, likes in SEREDRA_LIKE_KERNELS.items():
+            row = {}
+            for model, names in (("seredra", [new]), ("llama", likes)):
+                times = points[model][phase + "_kernels_us"]
+                us = sum(times.get(n, 0.0) for n in names)
+                name = next((n for n in names if n in times), None)
+                if not us or name is None:
+                    continue
+                w = work(name, rows, keys_sum, phase == "prefill")
+                row[model] = {"us": round(us, 1)}
+                if w:
+                    row[model]["share_of_peak"] = round(max(w[0] / (us * 1e-6) / (HBM_PEAK_GBS * 1e9),
+                                                            w[1] / (us * 1e-6) / PEAK_FLOPS["bf16"]), 4)
+            if "seredra" in row:
+                table[f"{phase}: {new}"] = row
+    return table
+
+
+def seredra_run(args) -> int:
+    T, batch, context = 2048, args.batch, args.context
+    out = {"metric": "Seredra beside the llama decoder at equal sizes: prefill tok/s (one prompt of 2048 tokens) and "
+                     f"decode tok/s (batch {batch}, context {context})", "unit": "tok/s", "n_gpus": 1,
+           "dtype": args.dtype, "data": "synthetic: random N(0, 0.02) weights, uniform random token ids",
+           "config": {"layers": "convolution attention + dense, retention + experts, (attention | selective scan) + "
+                                "dense, borrowing attention + experts",
+                      "experts": SEREDRA_EXPERTS, "top": SEREDRA_TOP, "states": SEREDRA_STATES, "taps": SEREDRA_TAPS,
+                      "page_tokens": 16},
+           "sizes": {}}
+    for size in args.design_sizes.split(","):
+        cfgs = seredra_configs(size, context)
+        points = {m: design_point(c, args.dtype, batch, context, args.steps, args.warmup, T) for m, c in cfgs.items()}
+        out["sizes"][size] = {
+            "shape": dict(zip(("width", "heads", "kv_heads", "head_size", "ff", "vocab"), DESIGN_SIZES[size])),
+            **points,
+            "prefill_seredra_over_llama": round(points["seredra"]["prefill_tok_s"] / points["llama"]["prefill_tok_s"], 3),
+            "decode_seredra_over_llama": round(points["seredra"]["decode_tok_s"] / points["llama"]["decode_tok_s"], 3),
+            "like_kernels": seredra_rooflines(size, batch, context, T, points)}
+    print(json.dumps(out), flush=True)
+    return 0
+
+
 def design_point(cfg_json, dtype, batch, context, steps, warmup, T):
     """Prefill tok/s (one prompt of T tokens in one step), decode tok/s (batch x context, graphs) and the time of
     every kernel in an eager prefill step and an eager decode step of one model."""
@@ -846,7 +981,7 @@ def main() -> int:
                     help="for profiling: only the decode steps at --batch (as --no-points), only the 2,048-token "
                          "prefill (prints its figures as the line's value), or only the sampler over the preset's "
                          "vocabulary (microseconds a step's rows take on the GPU and on the host)")
-    ap.add_argument("--design", choices=["risizen", "gulidra", "lesarax"], default=None,
+    ap.add_argument("--design", choices=["risizen", "gulidra", "lesarax", "seredra"], default=None,
                     help="instead of the default workload: the named design beside the llama decoder at equal sizes "
                          "(--design-sizes), prefill and decode throughput and the times of their like kernels")
     ap.add_argument("--design-sizes", default="1b,8b", help="with --design: sizes of the comparison, of " + ",".join(DESIGN_SIZES))
@@ -869,6 +1004,8 @@ def main() -> int:
         return gulidra_run(args)
     if args.design == "lesarax":
         return lesarax_run(args)
+    if args.design == "seredra":
+        return seredra_run(args)
     if args.design:
         return design_run(args)
     if args.kernel_times:

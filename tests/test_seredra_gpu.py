@@ -302,15 +302,19 @@ def test_retention_with_rotation_over_two_steps_and_the_norm_of_every_head(H, dk
         close(state[i].cpu().numpy(), S, "float32" if dtype == "float32" else "bfloat16", f"state {i}", rel=0.01)
 
 
-@pytest.mark.parametrize("C, N, taps", [(20, 5, 4), (256, 16, 4), (72, 8, 3), (8, 1, 1), (40, 100, 2), (130, 64, 5)])
+@pytest.mark.parametrize("C, N, taps, lens1, lens2", [
+    (20, 5, 4, [70, 3, 1], [1, 2, 22]), (256, 16, 4, [70, 3, 1], [1, 2, 22]), (72, 8, 3, [70, 3, 1], [1, 2, 22]),
+    (8, 1, 1, [70, 3, 1], [1, 2, 22]), (40, 100, 2, [70, 3, 1], [1, 2, 22]), (130, 64, 5, [70, 3, 1], [1, 2, 22]),
+    (96, 16, 4, [333, 64, 128], [65, 1, 200]), (50, 33, 3, [129, 1, 5], [1, 1, 1])])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_selective_scan_and_its_convolution_over_two_steps(C, N, taps, dtype):
-    """The convolution with its bias and silu, then the scan, with the last inputs and the state carried from a step of
-    portions of 70, 3 and 1 rows into a step of 1, 2 and 22 rows."""
+def test_selective_scan_and_its_convolution_over_two_steps(C, N, taps, lens1, lens2, dtype):
+    """The convolution with its bias and silu, then the scan, with the last inputs and the state carried from one step
+    of three portions into the next: portions of a row, of fewer rows than taps, of more rows than a chunk of the
+    kernel that takes the chunks of a portion side by side, ending on a chunk's edge and one row behind it; a step of
+    single rows only."""
     from allpaca_amd.kernels import ops
     rng = np.random.default_rng(C + N + taps)
     tdt = DTYPES[dtype]
-    lens1, lens2 = [70, 3, 1], [1, 2, 22]
     total = [a + b for a, b in zip(lens1, lens2)]
     xz = [bf(rng.normal(size=(L, 2 * C))) for L in total]
     dt = [np.float32(rng.normal(size=(L, C))) for L in total]
