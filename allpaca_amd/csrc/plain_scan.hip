@@ -49,6 +49,78 @@ __global__ void conv_channels_kernel(const void* __restrict__ x, int x_dtype, in
   store_f(out, out_dtype, (size_t)r * ldo + c, activate(acc, act));
 }
 
+// The same for bfloat16 rows, 8 consecutive channels a thread on 16-byte accesses (C, the row strides and the addresses
+// multiples of 8 elements), ROWS consecutive rows a block: a thread keeps its channels' taps in registers for all of
+// them, and a row that follows its predecessor in the same segment takes over that row's inputs and loads one more.
+// The same sums in the same order as the kernel above.
+template <int TAPS, int ROWS>
+__global__ __launch_bounds__(256) void conv_channels_bf16x8_kernel(
+    const bf16_t* __restrict__ x, int ldx, int n_rows, int C, const float* __restrict__ w,
+    const float* __restrict__ bias, const float* __restrict__ state, const int* __restrict__ row_seg,
+    const int* __restrict__ seg_row0, const int* __restrict__ slots, int act, bf16_t* __restrict__ out, int ldo) {
+  const int c = (blockIdx.y * 256 + threadIdx.x) * 8;
+  if (c >= C) return;
+  float wt[8][TAPS], b[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+#pragma unroll
+    for (int j = 0; j < TAPS; ++j) wt[e][j] = w[(size_t)(c + e) * TAPS + j];
+    b[e] = bias ? bias[c + e] : 0.f;
+  }
+  float u[TAPS][8];                               // the inputs of the row and of its TAPS - 1 predecessors, oldest first
+  int seg_before = -1;
+  for (int rr = 0; rr < ROWS; ++rr) {
+    const int r = blockIdx.x * ROWS + rr;
+    if (r >= n_rows) return;
+    const int seg = row_seg[r];
+    const int i_in_seg = r - seg_row0[seg];
+    auto load_input = [&](int j) {
+      const int back = TAPS - 1 - j;
+      if (back <= i_in_seg) {
+        const uint4 v = *reinterpret_cast<const uint4*>(x + (size_t)(r - back) * ldx + c);
+        const uint32_t p[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          u[j][2 * k] = __uint_as_float(p[k] << 16);
+          u[j][2 * k + 1] = __uint_as_float(p[k] & 0xffff0000u);
+        }
+      } else {
+        const float* sp = state + ((size_t)slots[seg] * (TAPS - 1) + (TAPS - 1 - (back - i_in_seg))) * C + c;
+        const float4 a = *reinterpret_cast<const float4*>(sp), d = *reinterpret_cast<const float4*>(sp + 4);
+        u[j][0] = a.x; u[j][1] = a.y; u[j][2] = a.z; u[j][3] = a.w;
+        u[j][4] = d.x; u[j][5] = d.y; u[j][6] = d.z; u[j][7] = d.w;
+      }
+    };
+    if (rr > 0 && seg == seg_before) {            // the row before is this row's predecessor
+#pragma unroll
+      for (int j = 0; j + 1 < TAPS; ++j)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) u[j][e] = u[j + 1][e];
+      load_input(TAPS - 1);
+    } else {
+#pragma unroll
+      for (int j = 0; j < TAPS; ++j) load_input(j);
+    }
+    seg_before = seg;
+    uint32_t o[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      float v[2];
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const int e = 2 * k + h;
+        float acc = 0.f;
+#pragma unroll
+        for (int j = 0; j < TAPS; ++j) acc = fmaf(wt[e][j], u[j][e], acc);     // oldest first
+        if (bias) acc += b[e];
+        v[h] = activate(acc, act);
+      }
+      o[k] = pack_bf16x2(v[0], v[1]);
+    }
+    *reinterpret_cast<uint4*>(out + (size_t)r * ldo + c) = uint4{o[0], o[1], o[2], o[3]};
+  }
+}
+
 // ---------------------------------------------------------------------------
 // Selective scan.  Per channel c with N states, over the rows of a segment in order:
 //   dt = softplus(dt_raw[t][c] + dt_bias[c])
@@ -153,6 +225,27 @@ APC_EXPORT int apc_conv_channels(const void* x, int x_dtype, int ldx, int n_rows
   if (C <= 0 || ldx < C || ldo < C || taps < 1 || !w || act < 0 || act > 3 || !row_seg || !seg_row0) return APC_ERR_BAD_ARG;
   if (taps > 1 && (!state || !slots)) return APC_ERR_BAD_ARG;
   if (taps > SCAN_MAX_TAPS || ceil_div(C, 256) > 65535) return APC_ERR_UNSUPPORTED;
+  if (x_dtype == APC_BF16 && out_dtype == APC_BF16 && taps <= 4 && C % 8 == 0 && ldx % 8 == 0 && ldo % 8 == 0 &&
+      !((uintptr_t)x & 15u) && !((uintptr_t)out & 15u) && !((uintptr_t)state & 15u)) {
+    const int rows_a_block = n_rows >= 512 ? 8 : 1;
+    const dim3 grid(ceil_div(n_rows, rows_a_block), ceil_div(C / 8, 256));
+#define CC_LAUNCH(TAPS_)                                                                                             \
+  do {                                                                                                               \
+    if (rows_a_block == 8)                                                                                           \
+      hipLaunchKernelGGL((conv_channels_bf16x8_kernel<TAPS_, 8>), grid, dim3(256), 0, stream, (const bf16_t*)x, ldx,  \
+                         n_rows, C, w, bias, state, row_seg, seg_row0, slots, act, (bf16_t*)out, ldo);               \
+    else                                                                                                             \
+      hipLaunchKernelGGL((conv_channels_bf16x8_kernel<TAPS_, 1>), grid, dim3(256), 0, stream, (const bf16_t*)x, ldx,  \
+                         n_rows, C, w, bias, state, row_seg, seg_row0, slots, act, (bf16_t*)out, ldo);               \
+  } while (0)
+    if (taps == 1) CC_LAUNCH(1);
+    else if (taps == 2) CC_LAUNCH(2);
+    else if (taps == 3) CC_LAUNCH(3);
+    else CC_LAUNCH(4);
+#undef CC_LAUNCH
+    APC_LAUNCH_CHECK();
+    return 0;
+  }
   hipLaunchKernelGGL(conv_channels_kernel, dim3(n_rows, ceil_div(C, 256)), dim3(256), 0, stream, x, x_dtype, ldx, C, w,
                      bias, taps, state, row_seg, seg_row0, slots, act, out, out_dtype, ldo);
   APC_LAUNCH_CHECK();

@@ -9,8 +9,9 @@
 //   outputs    every chunk again from the state in front of it: y_t = sum_n S_t[n] C_t[n] + D x_t, times silu(z_t)
 // All arithmetic is float32 (exponentials through the hardware's base-2 instruction); x, z and the output are
 // bfloat16 rows, the step sizes, B and C float32 rows.  A group of LPC lanes (a power of two) holds a channel's
-// states, a lane up to 16 of them in registers; with 16 states or fewer a thread is a channel, and B and C of a row
-// are the same addresses for the whole wave.  Steps whose segments are all short (decoded rows) stay on the kernel
+// states, a lane up to 16 of them in registers; with 16 states or fewer a thread is a channel.  B and C of a chunk's
+// rows, which every thread of a block reads, are put into LDS once a block (where they fit 32 KiB), and with exactly 16
+// states a thread reads them four at a time without a test of the state's number.  Steps whose segments are all short (decoded rows) stay on the kernel
 // that walks row by row, which reads and writes the state once.
 #include "mfma.h"
 #include <math.h>
@@ -24,19 +25,25 @@ constexpr float LOG2E_F = 1.4426950408889634f;
 __device__ __forceinline__ float softplus_f(float z) { return z > 20.f ? z : log1pf(__expf(z)); }
 __device__ __forceinline__ float silu_fast(float z) { return z / (1.0f + __expf(-z)); }
 
-template <int MODE>   // 1: summaries, 2: outputs
+template <int MODE, bool FULL>   // MODE 1: summaries, 2: outputs; FULL: 16 states a channel, a thread a channel
 __global__ __launch_bounds__(256) void scan_chunk_kernel(
     const bf16_t* __restrict__ x, int ldx, const float* __restrict__ dt_raw, int lddt,
     const float* __restrict__ dt_bias, const float* __restrict__ A, const float* __restrict__ bc, int ldbc,
     const float* __restrict__ Dw, const bf16_t* __restrict__ z, int ldz, float* __restrict__ ws,
     float* __restrict__ sumdt, int channels, int N, int lpc, const int* __restrict__ chunks,
-    const int* __restrict__ seg_row0, const int* __restrict__ seg_rows, bf16_t* __restrict__ out, int ldo) {
+    const int* __restrict__ seg_row0, const int* __restrict__ seg_rows, bf16_t* __restrict__ out, int ldo,
+    int staged) {
+  extern __shared__ float bcs[];                // [rows of the chunk][2 N], if `staged`
   const int chunk = blockIdx.y;
   const int seg = chunks[2 * chunk], in_seg = chunks[2 * chunk + 1];
   const int gid = blockIdx.x * 256 + threadIdx.x;
   const int c = gid / lpc, l = gid % lpc;
-  if (c >= channels) return;                    // (whole groups leave together: lpc divides 256)
   const int r0 = seg_row0[seg] + in_seg, n_rows = min(CHUNK, seg_rows[seg] - in_seg);
+  if (staged) {
+    for (int i = threadIdx.x; i < n_rows * 2 * N; i += 256) bcs[i] = bc[(size_t)(r0 + i / (2 * N)) * ldbc + i % (2 * N)];
+    __syncthreads();
+  }
+  if (c >= channels) return;                    // (whole groups leave together: lpc divides 256)
   float* w = ws + ((size_t)chunk * channels + c) * N;
   float s[NS], a2[NS];
 #pragma unroll
@@ -58,14 +65,32 @@ __global__ __launch_bounds__(256) void scan_chunk_kernel(
     }
     const float dx = dt * xv;
     total += dt;
-    const float* b = bc + r * ldbc;
+    const float* b = staged ? bcs + (size_t)t * 2 * N : bc + r * ldbc;
     float y = 0.f;
+    if (FULL) {
 #pragma unroll
-    for (int e = 0; e < NS; ++e) {
-      const int n = l + e * lpc;
-      if (n < N) {
-        s[e] = fmaf(__builtin_amdgcn_exp2f(dt * a2[e]), s[e], dx * b[n]);
-        if (MODE == 2) y = fmaf(s[e], b[N + n], y);
+      for (int e4 = 0; e4 < NS / 4; ++e4) {
+        const float4 bv = *reinterpret_cast<const float4*>(b + 4 * e4);
+        const float bb[4] = {bv.x, bv.y, bv.z, bv.w};
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+          s[4 * e4 + k] = fmaf(__builtin_amdgcn_exp2f(dt * a2[4 * e4 + k]), s[4 * e4 + k], dx * bb[k]);
+        if (MODE == 2) {
+          const float4 cv = *reinterpret_cast<const float4*>(b + NS + 4 * e4);
+          y = fmaf(s[4 * e4], cv.x, y);
+          y = fmaf(s[4 * e4 + 1], cv.y, y);
+          y = fmaf(s[4 * e4 + 2], cv.z, y);
+          y = fmaf(s[4 * e4 + 3], cv.w, y);
+        }
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < NS; ++e) {
+        const int n = l + e * lpc;
+        if (n < N) {
+          s[e] = fmaf(__builtin_amdgcn_exp2f(dt * a2[e]), s[e], dx * b[n]);
+          if (MODE == 2) y = fmaf(s[e], b[N + n], y);
+        }
       }
     }
     if (MODE == 2) {
@@ -135,16 +160,27 @@ APC_EXPORT int apc_selective_scan_bf16(const void* x, int ldx, const float* dt_r
   const long threads = (long)channels * lpc;
   if (n_chunks > 65535 || n_segs > 65535 || (threads + 255) / 256 > 0x7fffffffL) return APC_ERR_UNSUPPORTED;
   const dim3 grid((unsigned)((threads + 255) / 256), n_chunks);
-  hipLaunchKernelGGL(scan_chunk_kernel<1>, grid, dim3(256), 0, stream, (const bf16_t*)x, ldx, dt_raw, lddt, dt_bias, A,
-                     bc, ldbc, Dw, (const bf16_t*)z, ldz, ws, sumdt, channels, N, lpc, chunks, seg_row0, seg_rows,
-                     (bf16_t*)out, ldo);
-  APC_LAUNCH_CHECK();
+  // B and C of a chunk's rows in LDS (rows of the staged copy are 2 N floats: 16-byte reads need N a multiple of 2)
+  const size_t lds = (size_t)CHUNK * 2 * N * sizeof(float);
+  const int staged = lds <= 32 * 1024 ? 1 : 0;
+  const bool full = N == NS && staged;
+#define SCAN_LAUNCH(MODE_)                                                                                            \
+  do {                                                                                                                \
+    if (full)                                                                                                         \
+      hipLaunchKernelGGL((scan_chunk_kernel<MODE_, true>), grid, dim3(256), lds, stream, (const bf16_t*)x, ldx, dt_raw, \
+                         lddt, dt_bias, A, bc, ldbc, Dw, (const bf16_t*)z, ldz, ws, sumdt, channels, N, lpc, chunks,    \
+                         seg_row0, seg_rows, (bf16_t*)out, ldo, staged);                                              \
+    else                                                                                                              \
+      hipLaunchKernelGGL((scan_chunk_kernel<MODE_, false>), grid, dim3(256), staged ? lds : 0, stream,                \
+                         (const bf16_t*)x, ldx, dt_raw, lddt, dt_bias, A, bc, ldbc, Dw, (const bf16_t*)z, ldz, ws,      \
+                         sumdt, channels, N, lpc, chunks, seg_row0, seg_rows, (bf16_t*)out, ldo, staged);              \
+    APC_LAUNCH_CHECK();                                                                                               \
+  } while (0)
+  SCAN_LAUNCH(1);
   hipLaunchKernelGGL(scan_states_kernel, dim3(ceil_div(channels * N, 256), n_segs), dim3(256), 0, stream, ws, sumdt, A,
                      state, seg_chunks, slots, channels, N);
   APC_LAUNCH_CHECK();
-  hipLaunchKernelGGL(scan_chunk_kernel<2>, grid, dim3(256), 0, stream, (const bf16_t*)x, ldx, dt_raw, lddt, dt_bias, A,
-                     bc, ldbc, Dw, (const bf16_t*)z, ldz, ws, sumdt, channels, N, lpc, chunks, seg_row0, seg_rows,
-                     (bf16_t*)out, ldo);
-  APC_LAUNCH_CHECK();
+  SCAN_LAUNCH(2);
+#undef SCAN_LAUNCH
   return 0;
 }

@@ -305,7 +305,8 @@ def test_retention_with_rotation_over_two_steps_and_the_norm_of_every_head(H, dk
 @pytest.mark.parametrize("C, N, taps, lens1, lens2", [
     (20, 5, 4, [70, 3, 1], [1, 2, 22]), (256, 16, 4, [70, 3, 1], [1, 2, 22]), (72, 8, 3, [70, 3, 1], [1, 2, 22]),
     (8, 1, 1, [70, 3, 1], [1, 2, 22]), (40, 100, 2, [70, 3, 1], [1, 2, 22]), (130, 64, 5, [70, 3, 1], [1, 2, 22]),
-    (96, 16, 4, [333, 64, 128], [65, 1, 200]), (50, 33, 3, [129, 1, 5], [1, 1, 1])])
+    (96, 16, 4, [333, 64, 128], [65, 1, 200]), (50, 33, 3, [129, 1, 5], [1, 1, 1]),
+    (64, 16, 4, [601, 3, 70], [70, 519, 1]), (24, 4, 2, [515, 2, 1], [3, 2, 600])])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_selective_scan_and_its_convolution_over_two_steps(C, N, taps, lens1, lens2, dtype):
     """The convolution with its bias and silu, then the scan, with the last inputs and the state carried from one step
