@@ -112,15 +112,17 @@ __global__ __launch_bounds__(256) void rotary_pages_bf16_kernel(
   }
 }
 
-// One wave a (row, head): heads 0 .. H-1 are query heads, H .. H+G-1 keys (and their values).  d <= 512.
+// A group of `lph` lanes (a power of two from 8 on, at least a head's pieces) a (row, head), 256 / lph heads a block:
+// heads 0 .. H-1 are query heads, H .. H+G-1 keys (and their values).  d <= 512.
 __global__ __launch_bounds__(256) void rotary_pages_norm_bf16_kernel(
     const bf16_t* q, int ldq, int q_off, int H, int dq, int q_rot0, bf16_t* q_out, int ldqo,     // (q_out may be q)
     const bf16_t* __restrict__ ka, int ldka, int ka_off, int dk, int k_rot0, const bf16_t* __restrict__ v, int ldv,
     int v_off, int dv, int G, int rot, const float* __restrict__ cos_sin, const int* __restrict__ positions,
     const int* __restrict__ row_seg, const int* __restrict__ block_table, int max_blocks, bf16_t* __restrict__ cache,
-    int P, int with_values, const float* __restrict__ q_norm_w, const float* __restrict__ k_norm_w, float eps) {
-  const int r = blockIdx.x, hh = blockIdx.y * 4 + threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
-  if (hh >= H + G) return;
+    int P, int with_values, const float* __restrict__ q_norm_w, const float* __restrict__ k_norm_w, float eps,
+    int lph) {
+  const int r = blockIdx.x, hh = blockIdx.y * (256 / lph) + threadIdx.x / lph, lane = threadIdx.x % lph;
+  if (hh >= H + G) return;                      // (whole groups leave together; a wave holds whole groups)
   const bool is_q = hh < H;
   const int g = hh - H;
   const int d = is_q ? dq : dk, rot0 = is_q ? q_rot0 : k_rot0, half = rot / 2;
@@ -138,7 +140,7 @@ __global__ __launch_bounds__(256) void rotary_pages_norm_bf16_kernel(
   float ss = 0.f;
 #pragma unroll
   for (int i = 0; i < 8; ++i) ss = fmaf(x.v[i], x.v[i], ss);
-  ss = wave_sum(ss);
+  for (int o = lph / 2; o > 0; o >>= 1) ss += __shfl_xor(ss, o, WAVE);
   if (nw) {
     const float inv = 1.0f / sqrtf(ss / (float)d + eps);
     if (on) {
@@ -268,7 +270,10 @@ APC_EXPORT int apc_rotary_pages_bf16(const void* q, int ldq, int q_off, int H, i
   const long items = (long)H * (dq / 8) + (long)G * ((da + db) / 8) + (apart ? 0 : (long)G * (dv / 8));
   if (items > 65535L * 256) return APC_ERR_UNSUPPORTED;
   const bool normed = q_norm_w || k_norm_w;
-  if (normed && (db || dq > 512 || da > 512 || dv > 512 || (H + G + 3) / 4 > 65535 || !aligned16(q_norm_w) ||
+  int lph = 8;                                  // lanes a head: its pieces of 8 elements, rounded up to a power of two
+  while (lph * 8 < dq || lph * 8 < da || lph * 8 < dv) lph *= 2;
+  const int heads_a_block = 256 / (lph > 64 ? 64 : lph);
+  if (normed && (db || lph > 64 || (H + G + heads_a_block - 1) / heads_a_block > 65535 || !aligned16(q_norm_w) ||
                  !aligned16(k_norm_w)))
     return APC_ERR_UNSUPPORTED;
   if (apart) {
@@ -278,10 +283,12 @@ APC_EXPORT int apc_rotary_pages_bf16(const void* q, int ldq, int q_off, int H, i
     APC_LAUNCH_CHECK();
   }
   if (normed) {
-    hipLaunchKernelGGL(rotary_pages_norm_bf16_kernel, dim3(n_rows, (unsigned)((H + G + 3) / 4)), dim3(256), 0, stream,
+    hipLaunchKernelGGL(rotary_pages_norm_bf16_kernel,
+                       dim3(n_rows, (unsigned)((H + G + heads_a_block - 1) / heads_a_block)), dim3(256), 0, stream,
                        (const bf16_t*)q, ldq, q_off, H, dq, q_rot0, (bf16_t*)q_out, ldqo, (const bf16_t*)ka, ldka,
                        ka_off, da, k_rot0, (const bf16_t*)v, ldv, v_off, dv, G, rot, cos_sin, positions, row_seg,
-                       block_table, max_blocks, (bf16_t*)cache, page_tokens, apart ? 0 : 1, q_norm_w, k_norm_w, norm_eps);
+                       block_table, max_blocks, (bf16_t*)cache, page_tokens, apart ? 0 : 1, q_norm_w, k_norm_w, norm_eps,
+                       lph);
     APC_LAUNCH_CHECK();
     return 0;
   }

@@ -689,7 +689,8 @@ SEREDRA_LIKE_KERNELS = {
     "apc_attention_masked_decode_bf16": ["apc_attention_decode_bf16"],
     "apc_linear_attention_bf16": ["apc_attention_prefill_bf16"],
     "apc_linear_attention": ["apc_attention_decode_bf16"],
-    "apc_selective_scan": ["apc_attention_prefill_bf16", "apc_attention_decode_bf16"],
+    "apc_selective_scan_bf16": ["apc_attention_prefill_bf16"],
+    "apc_selective_scan": ["apc_attention_decode_bf16"],
     "apc_conv_channels": ["apc_rope_kv_write_bf16", "apc_rope_kv_write"],
     "apc_routed_experts_bf16": ["apc_gemm_swiglu_bf16", "apc_skinny_swiglu_bf16", "apc_skinny_swiglu_pre_bf16"],
     "apc_act_rows": [],
@@ -752,7 +753,8 @@ def seredra_rooflines(size, batch, context, T, points):
             return 0, rows * H * (2 * 32 * 2 * d + 2 * 2 * d * d)
         if name == "apc_linear_attention":       # the state of every row read and written
             return rows * H * d * d * 4 * 2, 0
-        if name == "apc_selective_scan":         # x, z, the step sizes read, y written; decoded rows: the state both ways
+        if name in ("apc_selective_scan", "apc_selective_scan_bf16"):
+            # x, z, the step sizes read, y written; decoded rows: the state both ways
             return rows * C * (2 + 2 + 4 + 2) + (0 if prefill else rows * C * N * 4 * 2), 0
         if name == "apc_conv_channels":
             return rows * C * (2 + 2), 0
