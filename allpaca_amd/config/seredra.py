@@ -191,7 +191,9 @@ def _attention(m: Mapping[str, Any], mw: str, i: int, layers: List[SeredraLayer]
     conv = m.get("conv")
     qt = m.get("q_temp")
     if qt is not None:
-        q = _obj(m, "q_temp", mw)
+        q = dict(_obj(m, "q_temp", mw))
+        if isinstance(q.get("every"), float) and q["every"].is_integer():      # (64.0 is 64)
+            q["every"] = int(q["every"])
         qt = (_num(q, "coef", mw + "q_temp."), _int(q, "every", mw + "q_temp."))
     mixer = SeredraAttention(heads=heads, kv_heads=kv, dim=_int(m, "dim", mw), vdim=_int(m, "vdim", mw),
                              scale=_num(m, "scale", mw), conv=0 if conv is None else _int(m, "conv", mw, least=0),
@@ -209,7 +211,9 @@ def _attention(m: Mapping[str, Any], mw: str, i: int, layers: List[SeredraLayer]
 
 
 def _parallel(m: Mapping[str, Any], mw: str) -> SeredraParallel:
-    l, lw = _obj(m, "left", mw), mw + "left."
+    l, lw = dict(_obj(m, "left", mw)), mw + "left."
+    if l.get("vdim") is None and l.get("dim") is not None:      # the values are the keys: one size for both
+        l["vdim"] = l["dim"]
     heads, kv = _heads(l, lw)
     dims, base = _rot(l, lw)
     sc = l["rot"].get("scaling")

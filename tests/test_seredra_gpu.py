@@ -432,20 +432,22 @@ ALONE = {
 }
 
 
-def folder_of(name):
+def folder_of(name, dtype="float32"):
+    """The model's folder; with "bfloat16" the one whose matrices are stored in 16 bits (the same values: the planted
+    weights are numbers that bfloat16 holds), which a bfloat16 run keeps in the matrix-core kernels' layout."""
     if name in ALONE:
         from helpers import tmp_root
         path = os.path.join(tmp_root(), "seredra_" + name)
         if not os.path.isdir(path):
             write_folder(path, *ALONE[name])
         return path
-    return model_folder(name)
+    return model_folder(name, dtype)
 
 
 def make_runner(name, dtype, page_tokens=4, num_pages=160, max_requests=3, poison=False, use_graphs=False):
     from allpaca_amd.engine.runner import ModelRunner
     from allpaca_amd.models import load_model
-    _, model = load_model(folder_of(name), DTYPES[dtype], DEV)
+    _, model = load_model(folder_of(name, dtype), DTYPES[dtype], DEV)
     return ModelRunner(model, page_tokens, num_pages, max_requests=max_requests, poison_free_pages=poison,
                        use_graphs=use_graphs)
 
@@ -524,6 +526,27 @@ def test_whole_prompts_decoding_and_portions(name, dtype, page_tokens):
     for cuts in ([2], [3, 2, 7, 1, 5], [6, 13, 2, 2, 66], [65, 1, 1, 2, 19, 3]):
         check(run_cut(runner, toks, cuts), name, toks, dtype, f"portions {cuts}")
     runner.cache.check()
+
+
+def test_a_bfloat16_run_is_on_the_matrix_core_kernels():
+    """A prompt portion and a decoded row of a model whose sizes the bfloat16 kernels take: the new mechanisms run on
+    them and not on the plain kernels they would otherwise fall back to."""
+    from allpaca_amd.engine.batch import Entry
+    from allpaca_amd.kernels import lib as klib
+    toks = tokens_for("SB", 70, 5)
+    runner = make_runner("SB", "bfloat16", page_tokens=16)
+    runner.admit("s")
+    with klib.timing() as t:
+        runner.step([Entry("s", toks[:69], [68])])
+        runner.step([Entry("s", toks[69:], [0])])
+    used = set(t.totals())
+    runner.release("s")
+    for name in ("apc_conv_heads_bf16", "apc_attention_masked_prefill_bf16", "apc_attention_masked_decode_bf16",
+                 "apc_rotary_pages_bf16", "apc_linear_rotate_bf16", "apc_linear_attention_bf16",
+                 "apc_selective_scan_bf16", "apc_routed_experts_bf16", "apc_gemm_bf16"):
+        assert name in used, (name, sorted(used))
+    for name in ("apc_conv_heads", "apc_masked_attention_plain", "apc_rotary_pages", "apc_routed_glu", "apc_gemm_plain"):
+        assert name not in used, (name, sorted(used))
 
 
 def test_cuttings_agree_to_the_bit_in_32_bit():
