@@ -87,9 +87,9 @@ TINY_SC = _model(50, 32, 1.0, 1e-6, [
 #    experts, two borrowers of one owner, whole heads rotated
 TINY_SD = _model(300, 96, 9.0, 1e-6, [
     _layer(_att(6, 2, 24, 40, 0.2, conv=3, q_temp=(0.3, 5)), _moe(72, 10, 4)),
-    _layer(_ret(3, 40, 24, (0.96875, 0.9, 0.99), 40, 1000.0), _dense(200)),
+    _layer(_ret(3, 40, 24, (0.97, 0.9, 0.99), 40, 1000.0), _dense(200)),
     _layer(_att(6, 2, 24, 40, 0.15, conv=5, kv_from=0), None),
-    _layer(_par((6, 3, 40, 0.15, 40, 5000.0, 10.0, (2.0, 32, 4.0, 0.5)), (72, 8, 6, 3), 0.8, 0.5), _dense(104)),
+    _layer(_par((6, 3, 40, 0.15, 40, 5000.0, 10.0, (2.0, 32, 4.0, 0.5)), (72, 8, 6, 3), 0.9, 0.4), _dense(104)),
     _layer(_att(6, 2, 24, 40, 0.25, kv_from=0), _moe(24, 3, 1))])
 
 CONFIGS = {"SA": (TINY_SA, 51), "SB": (TINY_SB, 52), "SC": (TINY_SC, 53), "SD": (TINY_SD, 54)}

@@ -160,7 +160,7 @@ def test_convolution_norm_over_the_whole_projection_and_query_temperature(H, G, 
 
 @pytest.mark.parametrize("H, G, dk, dv, P_, cap, bias", [(4, 2, 12, 12, 4, 0.0, True), (3, 3, 16, 14, 3, 2.5, False),
                                                          (8, 2, 64, 64, 16, 0.0, True), (8, 4, 32, 64, 16, 0.0, True),
-                                                         (6, 3, 96, 96, 16, 6.0, False), (4, 1, 128, 128, 16, 3.0, True),
+                                                         (12, 4, 96, 96, 16, 6.0, False), (4, 1, 128, 128, 16, 3.0, True),
                                                          (6, 2, 40, 24, 8, 0.0, True)])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_distance_penalty_and_soft_cap_over_pages_with_one_key_that_stands_out(H, G, dk, dv, P_, cap, bias, dtype):
@@ -214,7 +214,7 @@ def test_distance_penalty_and_soft_cap_over_pages_with_one_key_that_stands_out(H
 
 @pytest.mark.parametrize("H, G, dk, rot, P_, scaling", [(4, 2, 12, 4, 3, (3.0, 16, 8.0, 1.0)), (8, 2, 64, 32, 16, (4.0, 64, 16.0, 2.0)),
                                                         (3, 3, 16, 16, 8, None), (2, 1, 40, 0, 4, None),
-                                                        (6, 3, 96, 96, 16, (2.0, 128, 32.0, 1.0)), (4, 4, 128, 64, 16, None)])
+                                                        (12, 4, 96, 64, 16, (5.0, 128, 16.0, 2.0)), (4, 4, 128, 64, 16, None)])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_head_norms_rotation_under_a_frequency_rule_and_values_that_stay_as_projected(H, G, dk, rot, P_, scaling, dtype):
     """One projected row holds q and k.  Every head is normed with weights all heads share, then rotated; k goes into
